@@ -39,7 +39,7 @@ class LayerGroup:
     space: int
     owners: list[int]                 # run-order indices of the layer runs whose caches live here
     k_pool: torch.Tensor              # [len(owners), pool pages, kv_heads, pool page size, head_dim]
-    v_pool: torch.Tensor              # [len(owners), pool pages, kv_heads, head_dim, pool page size]
+    v_pool: torch.Tensor              # [len(owners), pool pages, kv_heads, value_dim, pool page size]
 
 
 def plan_spaces(kv_specs: list[KVSpec]) -> tuple[list[tuple[KVSpec, int]], int]:
@@ -60,7 +60,7 @@ def bytes_per_page(cache_plan, page_size: int, dtype: torch.dtype, space: int = 
     """Bytes that one page id of `space` occupies over all layers (keys and values)."""
     assigned, _ = plan_spaces([e.kv for e in cache_plan])
     lookup = dict((kv, s) for kv, s in assigned)
-    return sum(2 * page_size * e.kv.num_kv_heads * e.kv.head_dim * dtype.itemsize
+    return sum(page_size * e.kv.num_kv_heads * (e.kv.head_dim + e.kv.v_dim) * dtype.itemsize
                for e in cache_plan if lookup[e.kv] == space)
 
 
@@ -93,7 +93,7 @@ class KVStorage:
         for kv, s in assigned:
             owners = [e.owner for e in cache_plan if e.kv == kv]
             k_shape = (len(owners), pages[s] * self.pages_per_entry, kv.num_kv_heads, self.pool_page, kv.head_dim)
-            v_shape = (len(owners), pages[s] * self.pages_per_entry, kv.num_kv_heads, kv.head_dim, self.pool_page)
+            v_shape = (len(owners), pages[s] * self.pages_per_entry, kv.num_kv_heads, kv.v_dim, self.pool_page)
             group = LayerGroup(kv, s, owners, torch.zeros(k_shape, dtype=dtype, device=self.device),
                                torch.zeros(v_shape, dtype=dtype, device=self.device))
             for j, owner in enumerate(owners):

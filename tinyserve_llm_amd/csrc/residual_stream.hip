@@ -1,0 +1,134 @@
+// A residual stream kept in 32-bit floats whatever the storage type of the activations around it:
+//   * token rows of the embedding table into the stream,
+//   * the stream's update x += mult * (a + b + bias) by what two parallel branches (or one) have made,
+//     with up to two weighted RMS norms of the updated row on the way out (both share the row's mean
+//     square, which is taken once), or the norms alone, or the norms of a few picked rows,
+//   * a bias and an activation between two projections of a dense feed-forward.
+// Sums, mean squares, roots and scalings are 32-bit; what leaves for a projection is rounded to the
+// activations' storage type only at the store. Every row is worked on by one workgroup and by itself:
+// a row's result does not depend on the rows beside it.
+#include "common.h"
+
+#define RS_THREADS 256
+
+// value of element i of a row stored as float (code 0) or bfloat16 (code 1)
+static __device__ __forceinline__ float rs_load(const void* p, int code, int64_t i) {
+  return code == 0 ? ((const float*)p)[i] : bf2f(((const bf16_t*)p)[i]);
+}
+static __device__ __forceinline__ void rs_store(void* p, int code, int64_t i, float v) {
+  if (code == 0) ((float*)p)[i] = v;
+  else ((bf16_t*)p)[i] = f2bf(v);
+}
+
+static __device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
+  __syncthreads();                 // (scratch may still be read from a sum before)
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < RS_THREADS / TS_WAVE; ++w) total += scratch[w];
+  return total;
+}
+
+__global__ void __launch_bounds__(RS_THREADS)
+embedding_stream_kernel(float* __restrict__ out, const void* __restrict__ table, const int32_t* __restrict__ ids,
+                        int hidden, int code) {
+  const int64_t t = blockIdx.x;
+  const int64_t src = (int64_t)ids[t] * hidden;
+  for (int i = threadIdx.x; i < hidden; i += RS_THREADS) out[t * hidden + i] = rs_load(table, code, src + i);
+}
+
+extern "C" int ts_embedding_stream(float* out, const void* table, const int32_t* ids, int num_tokens, int hidden,
+                                   int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return TS_OK;
+  if (hidden <= 0) return TS_BAD_SHAPE;
+  if (dtype != 0 && dtype != 1) return TS_BAD_DTYPE;
+  embedding_stream_kernel<<<num_tokens, RS_THREADS, 0, stream>>>(out, table, ids, hidden, dtype);
+  return ts_check_launch();
+}
+
+// Row r of the grid: stream row t = rows ? rows[r] : r.
+//   update (a or b given; rows must be null): x[t] += mult * (a[t] + b[t] + bias), written back
+//   norms (h1 / h2 given): h[r] = x[t] / sqrt(mean(x[t]^2) + eps) * w, of the updated row
+__global__ void __launch_bounds__(RS_THREADS)
+stream_update_norm_kernel(float* __restrict__ x, const void* __restrict__ a, int a_code, const void* __restrict__ b,
+                          int b_code, const void* __restrict__ bias, int bias_code, float mult,
+                          void* __restrict__ h1, void* __restrict__ h2, int h_code, const void* __restrict__ w1,
+                          const void* __restrict__ w2, int w_code, float eps, const int32_t* __restrict__ rows,
+                          int width) {
+  __shared__ float scratch[RS_THREADS / TS_WAVE];
+  const int64_t r = blockIdx.x;
+  const int64_t t = rows ? rows[r] : r;
+  float* xr = x + t * width;
+  const bool update = a || b;
+  float squares = 0.f;
+  for (int i = threadIdx.x; i < width; i += RS_THREADS) {
+    float v = xr[i];
+    if (update) {
+      float add = 0.f;
+      if (a) add += rs_load(a, a_code, t * width + i);
+      if (b) add += rs_load(b, b_code, t * width + i);
+      if (bias) add += rs_load(bias, bias_code, i);
+      v = fmaf(mult, add, v);
+      xr[i] = v;
+    }
+    squares = fmaf(v, v, squares);
+  }
+  if (!h1 && !h2) return;
+  const float total = block_sum(squares, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += RS_THREADS) {
+    const float v = xr[i] * inv;       // (this thread's own elements, as it has just written them)
+    if (h1) rs_store(h1, h_code, r * width + i, v * rs_load(w1, w_code, i));
+    if (h2) rs_store(h2, h_code, r * width + i, v * rs_load(w2, w_code, i));
+  }
+}
+
+extern "C" int ts_stream_update_norm(float* x, const void* a, int a_dtype, const void* b, int b_dtype, const void* bias,
+                                     int bias_dtype, float mult, void* h1, void* h2, int h_dtype, const void* w1,
+                                     const void* w2, int w_dtype, float eps, const int32_t* rows, int num_rows, int width,
+                                     hipStream_t stream) {
+  if (num_rows <= 0) return TS_OK;
+  if (width <= 0 || !x || (rows && (a || b)) || (h1 && !w1) || (h2 && !w2)) return TS_BAD_SHAPE;
+  for (int code : {a_dtype, b_dtype, bias_dtype, h_dtype, w_dtype})
+    if (code != 0 && code != 1) return TS_BAD_DTYPE;
+  stream_update_norm_kernel<<<num_rows, RS_THREADS, 0, stream>>>(x, a, a_dtype, b, b_dtype, bias, bias_dtype, mult, h1, h2,
+                                                                 h_dtype, w1, w2, w_dtype, eps, rows, width);
+  return ts_check_launch();
+}
+
+// out[t, i] = act(in[t, i] + bias[i]); act 0: none, 1: relu squared, 2: gelu (tanh form), 3: silu
+static __device__ __forceinline__ float rs_activate(float z, int act) {
+  switch (act) {
+    case 1: { const float r = fmaxf(z, 0.f); return r * r; }
+    case 2: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    case 3: return z / (1.0f + expf(-z));
+    default: return z;
+  }
+}
+
+__global__ void __launch_bounds__(RS_THREADS)
+bias_activation_kernel(void* __restrict__ out, int out_code, const void* __restrict__ in, int in_code,
+                       const void* __restrict__ bias, int bias_code, int64_t total, int width, int act) {
+  for (int64_t idx = (int64_t)blockIdx.x * RS_THREADS + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * RS_THREADS) {
+    const int i = (int)(idx % width);
+    float z = rs_load(in, in_code, idx);
+    if (bias) z += rs_load(bias, bias_code, i);
+    rs_store(out, out_code, idx, rs_activate(z, act));
+  }
+}
+
+extern "C" int ts_bias_activation(void* out, int out_dtype, const void* in, int in_dtype, const void* bias, int bias_dtype,
+                                  int num_rows, int width, int act, hipStream_t stream) {
+  if (num_rows <= 0) return TS_OK;
+  if (width <= 0 || act < 0 || act > 3) return TS_BAD_SHAPE;
+  for (int code : {out_dtype, in_dtype, bias_dtype})
+    if (code != 0 && code != 1) return TS_BAD_DTYPE;
+  const int64_t total = (int64_t)num_rows * width;
+  int64_t blocks = (total + RS_THREADS - 1) / RS_THREADS;
+  if (blocks > 16384) blocks = 16384;
+  bias_activation_kernel<<<(unsigned)blocks, RS_THREADS, 0, stream>>>(out, out_dtype, in, in_dtype, bias, bias_dtype, total,
+                                                                     width, act);
+  return ts_check_launch();
+}

@@ -24,7 +24,7 @@ from tinyserve_llm_amd.engine.loading import as_dtype, load_model
 from tinyserve_llm_amd.engine.runner import ModelRunner, StepEntry
 
 REPLAY_PAGE_SIZE = 64
-MAX_LIVE = 16
+MAX_LIVE = 4        # state slots: requests that may be live at once
 
 
 class Replay:

@@ -41,12 +41,20 @@ class DecoderModel:
                 raise KeyError(f"block arrangement {ls.block!r} asks for the norms {lacking}; the layer names {sorted(ls.norms)}")
             self.layers.append(Layer(
                 mixer=base.make("mixer", ls.mixer), feed_forward=base.make("feed_forward", ls.feed_forward),
-                norms={name: base.make("norm", ps) for name, ps in ls.norms.items()}, block=ls.block))
+                norms={name: base.make("norm", ps) for name, ps in ls.norms.items()}, block=ls.block,
+                block_args=dict(ls.block_args)))
         self.final_norm = base.make("norm", spec.final_norm)
         self.position_encodings = {name: base.make("position_encoding", ps)
                                    for name, ps in spec.position_encodings.items()}
         sizes = dict(vocab_size=spec.vocab_size, hidden_size=spec.hidden_size, init=spec.embedding_init)
-        self.embedding = base.make("embedding", spec.embedding or PartSpec("table", sizes))
+        if spec.residual_dtype not in ("compute", "float32"):
+            raise ValueError(f"residual_dtype {spec.residual_dtype!r}: 'compute' or 'float32'")
+        if spec.residual_dtype == "float32":
+            unfit = sorted({ls.block for ls in spec.layers if not getattr(base.BLOCKS[ls.block], "keeps_stream", False)})
+            if unfit:
+                raise ValueError(f"a 32-bit residual stream needs block arrangements that keep it; {unfit} do not")
+        table_args = dict(sizes, float32_stream=True) if spec.residual_dtype == "float32" else sizes
+        self.embedding = base.make("embedding", spec.embedding or PartSpec("table", table_args))
         self.head = base.make("head", spec.head or PartSpec("projection", dict(sizes, tied=spec.tie_word_embeddings)))
         self.dtype: torch.dtype | None = None
         self.device: torch.device | None = None
@@ -64,7 +72,7 @@ class DecoderModel:
                 if owner.cache is not None:
                     raise ValueError(f"order[{i}] must name the entry that owns the cache, not a borrower")
                 a, b = self.layers[run.layer].mixer.kv_spec(), self.layers[owner.layer].mixer.kv_spec()
-                if a is None or b is None or (a.num_kv_heads, a.head_dim) != (b.num_kv_heads, b.head_dim):
+                if a is None or b is None or (a.num_kv_heads, a.head_dim, a.v_dim) != (b.num_kv_heads, b.head_dim, b.v_dim):
                     raise ValueError(f"order[{i}] and order[{run.cache}] cache rows of different shapes")
             elif not run.store and self.layers[run.layer].mixer.kv_spec() is not None:
                 raise ValueError(f"order[{i}] neither owns a cache to write nor names one to read")

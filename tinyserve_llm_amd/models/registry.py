@@ -59,7 +59,10 @@ def register_architecture(arch: Architecture) -> Architecture:
 
 
 def resolve(raw: Mapping[str, Any]) -> Architecture:
-    for name in raw.get("architectures") or []:
+    named = list(raw.get("architectures") or [])
+    if isinstance(raw.get("architecture"), str):       # (some configurations name theirs in one string)
+        named.append(raw["architecture"])
+    for name in named:
         if name in ARCHITECTURES:
             return ARCHITECTURES[name]
     model_type = raw.get("model_type")
@@ -67,7 +70,7 @@ def resolve(raw: Mapping[str, Any]) -> Architecture:
         if model_type in arch.model_types:
             return arch
     raise NotImplementedError(
-        f"architecture {raw.get('architectures')!r} / model_type {model_type!r} is not supported; "
+        f"architecture {named!r} / model_type {model_type!r} is not supported; "
         f"have {sorted(ARCHITECTURES)}")
 
 

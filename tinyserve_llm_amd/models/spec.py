@@ -20,6 +20,7 @@ class LayerSpec:
     feed_forward: PartSpec
     norms: Mapping[str, PartSpec]
     block: str = "pre_norm"
+    block_args: Mapping[str, object] = field(default_factory=dict)      # constants of the arrangement itself
 
     @classmethod
     def pre_norm(cls, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec, ff_norm: PartSpec) -> "LayerSpec":
@@ -77,6 +78,9 @@ class ModelSpec:
     tie_word_embeddings: bool = False
     eos_token_id: int = -1
     embedding_init: tuple[float, float] = (0.0, 0.02)
+    # "compute": the residual stream has the engine's storage type; "float32": it is kept in 32-bit
+    # floats whatever that type (`parts.stream.ResidualStream`; every block must declare `keeps_stream`)
+    residual_dtype: str = "compute"
     # what turns token ids into the first hidden rows, and the final rows into logits; None: a
     # plain table and a plain projection (tied to the table if `tie_word_embeddings`)
     embedding: PartSpec | None = None

@@ -73,6 +73,13 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_skinny_tiles": [i, i, i],
         "ts_peak_read": [p, ctypes.c_size_t, p, i, p],
         "ts_peak_mfma": [p, i, i, p],
+        "ts_embedding_stream": [p, p, p, i, i, i, p],
+        "ts_stream_update_norm": [p, p, i, p, i, p, i, f, p, p, i, p, p, i, f, p, i, i, p],
+        "ts_bias_activation": [p, i, p, i, p, i, i, i, i, p],
+        "ts_mingru_scan": [p, i, p, i, p, i, p, p, p, i, i, i, p],
+        "ts_qkv_finish": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, f, i, f, i, i64, i64, i64, i64, i64, i64, i64, i, i, p],
+        "ts_paged_attention_general": [p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, f, i, i,
+                                       i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
                                      i64, i64, i64, i64, p, i, p],
     }
@@ -1491,3 +1498,191 @@ def measure_peaks(read_bytes: int = 2 << 30, repeats: int = 5) -> dict[str, floa
     return {"read_GBps": data.numel() * 4 / read_s / 1e9,
             "mfma_bf16_TFLOPs": groups * 4 * iters * 4 * 2 * 16 * 16 * 32 / mfma_s / 1e12}
 
+
+
+# ---- a 32-bit residual stream, parallel branches, a dense feed-forward's bias and activation ----
+
+def embedding_stream(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[ids[t]] as float32 rows, whatever the table's storage type: the start of a
+    residual stream that is kept in 32-bit."""
+    _gpu(table, ids)
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [vocab, hidden]")
+    _need(ids.dtype == torch.int32 and ids.dim() == 1 and ids.is_contiguous(), "ids must be int32 [tokens]")
+    out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32, device=table.device)
+    _run("embedding_stream", library().ts_embedding_stream(_ptr(out), _ptr(table), _ptr(ids), ids.shape[0], table.shape[1],
+                                                           _code(table.dtype), _stream()))
+    return out
+
+
+def stream_update_norm(x: torch.Tensor, a: torch.Tensor | None = None, b: torch.Tensor | None = None,
+                       bias: torch.Tensor | None = None, mult: float = 1.0,
+                       weights: "tuple[torch.Tensor | None, torch.Tensor | None]" = (None, None), eps: float = 0.0,
+                       rows: torch.Tensor | None = None, out_dtype: torch.dtype = torch.float32
+                       ) -> "tuple[torch.Tensor | None, torch.Tensor | None]":
+    """The float32 stream x [tokens, width] takes x += mult * (a + b + bias) in place (a, b: what
+    parallel branches made, float32 or bfloat16, either may be None; bias [width] rides on them), and
+    for each given weight norm(x) * weight of the updated rows comes back in `out_dtype` (both norms
+    share the row's mean square). With `rows` (int32) nothing is updated and only those rows are
+    normalised, in that order."""
+    _gpu(x, a, b, bias, rows, *weights)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "the stream must be contiguous float32 [tokens, width]")
+    tokens, width = x.shape
+    for name, t in (("a", a), ("b", b)):
+        _need(t is None or (t.shape == x.shape and t.is_contiguous()), lambda: f"{name} must match the stream")
+    _need(bias is None or (bias.shape == (width,) and bias.is_contiguous() and (a is not None or b is not None)),
+          "a bias is [width] and rides on a branch")
+    _need(rows is None or (a is None and b is None), "picked rows are normalised, not updated")
+    n = tokens
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.dim() == 1 and rows.is_contiguous(), "rows must be int32")
+        n = rows.shape[0]
+    given = [w for w in weights if w is not None]
+    for w in given:
+        _need(w.shape == (width,) and w.is_contiguous() and w.dtype == given[0].dtype, "norm weights must be [width], of one type")
+    outs = [None if w is None else torch.empty((n, width), dtype=out_dtype, device=x.device) for w in weights]
+    _run("stream_update_norm", library().ts_stream_update_norm(
+        _ptr(x), _ptr(a), 0 if a is None else _code(a.dtype), _ptr(b), 0 if b is None else _code(b.dtype),
+        _ptr(bias), 0 if bias is None else _code(bias.dtype), float(mult), _ptr(outs[0]), _ptr(outs[1]), _code(out_dtype),
+        _ptr(weights[0]), _ptr(weights[1]), _code(given[0].dtype) if given else 0, float(eps), _ptr(rows), n, width, _stream()))
+    return outs[0], outs[1]
+
+
+ACTIVATIONS = {"none": 0, "relu2": 1, "gelu_tanh": 2, "silu": 3}
+
+
+def bias_activation(x: torch.Tensor, bias: torch.Tensor | None, activation: str, out_dtype: torch.dtype) -> torch.Tensor:
+    """act(x + bias) row by row, taken in 32-bit and stored as `out_dtype`. "relu2": the square of
+    relu; "gelu_tanh": 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))."""
+    _gpu(x, bias)
+    _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: one of {sorted(ACTIVATIONS)}")
+    _need(x.dim() == 2 and x.is_contiguous(), "the input must be contiguous [tokens, width]")
+    _need(bias is None or (bias.shape == (x.shape[1],) and bias.is_contiguous()), "the bias must be [width]")
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    _run("bias_activation", library().ts_bias_activation(
+        _ptr(out), _code(out_dtype), _ptr(x), _code(x.dtype), _ptr(bias), 0 if bias is None else _code(bias.dtype),
+        x.shape[0], x.shape[1], ACTIVATIONS[activation], _stream()))
+    return out
+
+
+# ---- minGRU ----
+
+MINGRU_STRETCH = 32       # tokens of a request's portion per wave from which the scan is cut into stretches
+MINGRU_MAX_WAVES = 16
+
+
+def mingru_waves(longest: int) -> int:
+    """Waves (stretches of a portion) that the scan gives the longest portion of a step."""
+    return max(1, min(MINGRU_MAX_WAVES, longest // MINGRU_STRETCH))
+
+
+def mingru_scan(zxg: torch.Tensor, bias: torch.Tensor | None, state: torch.Tensor, cu_seqlens: torch.Tensor,
+                state_slots: torch.Tensor, longest: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """The minGRU recurrence over a packed step: zxg [tokens, 3 width] holds the projected z | x | g
+    rows, bias [2 width] the biases of z and x; request s owns tokens cu_seqlens[s] .. cu_seqlens[s+1]
+    and the float32 state row state[state_slots[s]], which the step advances. Returns
+    S_t * silu(g_t) [tokens, width] in `out_dtype`. `longest`: the most tokens any request feeds."""
+    _gpu(zxg, bias, state, cu_seqlens, state_slots)
+    _need(zxg.dim() == 2 and zxg.shape[1] % 3 == 0 and zxg.is_contiguous(), "zxg must be contiguous [tokens, 3 width]")
+    width = zxg.shape[1] // 3
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == width and state.is_contiguous(),
+          lambda: f"the state must be contiguous float32 [slots, {width}]")
+    _need(bias is None or (bias.shape == (2 * width,) and bias.is_contiguous()), "the bias must be [2 width]")
+    num_seqs = state_slots.shape[0]
+    _need(state_slots.dtype == torch.int32 and state_slots.dim() == 1 and state_slots.is_contiguous(), "state_slots must be int32")
+    _need(cu_seqlens.dtype == torch.int32 and cu_seqlens.shape == (num_seqs + 1,) and cu_seqlens.is_contiguous(),
+          "cu_seqlens must be int32 [requests + 1]")
+    out = torch.empty((zxg.shape[0], width), dtype=out_dtype, device=zxg.device)
+    _run("mingru_scan", library().ts_mingru_scan(
+        _ptr(out), _code(out_dtype), _ptr(zxg), _code(zxg.dtype), _ptr(bias), 0 if bias is None else _code(bias.dtype),
+        _ptr(state), _ptr(cu_seqlens), _ptr(state_slots), num_seqs, width, mingru_waves(longest), _stream()))
+    return out
+
+
+# ---- attention with head norms, capped scores, a sink, and values of their own size ----
+
+def _check_cache_pair(k_cache: torch.Tensor, v_cache: torch.Tensor, dtype: torch.dtype, nkv: int, hd: int, vd: int) -> None:
+    """`_check_cache` for caches whose value rows have a size of their own."""
+    for name, c, size in (("key", k_cache, hd), ("value", v_cache, vd)):
+        _need(c.dim() == 4 and c.shape[2] == nkv and c.shape[3] == size,
+              lambda: f"{name} cache view must be [pages, page_size, {nkv}, {size}], got {tuple(c.shape)}")
+        _need(c.dtype == dtype, "cache and activations differ in storage type")
+        span = 1
+        for stride, extent in sorted(zip(c.stride(), c.shape)):
+            if extent > 1:
+                _need(stride >= span, lambda: f"{name} cache elements overlap")
+                span = stride * extent
+    _need(k_cache.shape[:3] == v_cache.shape[:3], "key and value caches differ in pages, slots or heads")
+    _need(k_cache.stride(3) == 1, "a key row must be contiguous in the key cache")
+
+
+def qkv_finish(qkv: torch.Tensor, freqs: torch.Tensor | None, positions: torch.Tensor, slots: torch.Tensor | None,
+               k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, num_heads: int, num_kv_heads: int,
+               head_dim: int, value_dim: int, out_dtype: torch.dtype, *, interleaved: bool = True,
+               qk_norm_eps: float | None = None, v_norm_eps: float | None = None) -> torch.Tensor:
+    """From a projected row q | k | v ([tokens, nh hd + nkv hd + nkv vd], float32 or `out_dtype`) to q
+    [tokens, nh, hd] and the cache slots of k and v, in `out_dtype`. `freqs` (float64 [rot / 2]): q and
+    k turn in their first rot dimensions by position * freqs[i], pair i being dimensions (2i, 2i+1) if
+    `interleaved`, else (i, i + rot/2). `qk_norm_eps` / `v_norm_eps`: each q and k head, and each value
+    head, is then divided by its root mean square (eps inside the root); None: not."""
+    _gpu(qkv, freqs, positions, slots, k_cache, v_cache)
+    T = qkv.shape[0]
+    row = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
+    _need(qkv.dim() == 2 and qkv.shape[1] == row and qkv.is_contiguous(), lambda: f"qkv must be contiguous [tokens, {row}]")
+    _need(qkv.dtype in (torch.float32, out_dtype), "the projected rows are float32 or of the output's type")
+    _need(0 < head_dim <= 256 and 0 < value_dim <= 256, "head sizes up to 256")
+    _need(positions.dtype == torch.int32 and positions.shape == (T,) and positions.is_contiguous(), "positions must be int32 [tokens]")
+    rot = 0
+    if freqs is not None:
+        _need(freqs.dtype == torch.float64 and freqs.dim() == 1 and freqs.is_contiguous() and 2 * freqs.shape[0] <= head_dim,
+              "frequencies must be float64 [rot / 2], rot up to head_dim")
+        rot = 2 * freqs.shape[0]
+    page_size, kst, vst = 1, (0, 0, 0), (0, 0, 0, 0)
+    if k_cache is not None:
+        _need(v_cache is not None and slots is not None, "a cache write needs k, v and the slots")
+        _need(slots.dtype == torch.int32 and slots.shape == (T,) and slots.is_contiguous(), "slots must be int32 [tokens]")
+        _check_cache_pair(k_cache, v_cache, out_dtype, num_kv_heads, head_dim, value_dim)
+        page_size, kst, vst = k_cache.shape[1], k_cache.stride()[:3], v_cache.stride()
+    q = torch.empty((T, num_heads, head_dim), dtype=out_dtype, device=qkv.device)
+    _run("qkv_finish", library().ts_qkv_finish(
+        _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(qkv), _ptr(freqs), _ptr(positions), _ptr(slots), T, num_heads,
+        num_kv_heads, head_dim, value_dim, rot, int(interleaved), int(qk_norm_eps is not None), float(qk_norm_eps or 0.0),
+        int(v_norm_eps is not None), float(v_norm_eps or 0.0), page_size, *kst, *vst, _code(qkv.dtype), _code(out_dtype),
+        _stream()))
+    return q
+
+
+def paged_attention_general(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                            seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, *, softcap: float = 0.0,
+                            sink: bool = False, window: int = 0, pages_per_entry: int = 1) -> torch.Tensor:
+    """Attention of each token (at its position, causal, optionally windowed) over its request's
+    pages, in 32-bit: score = q.k * scale, capped as softcap * tanh(score / softcap) if softcap > 0;
+    with `sink` the softmax has one more in its denominator (a key of score 0 without a value).
+    Value rows may differ in size from key rows: out [tokens, heads, value_dim]."""
+    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
+    _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
+    T, nh, hd = q.shape
+    nkv, vd = k_cache.shape[2], v_cache.shape[3]
+    _check_cache_pair(k_cache, v_cache, q.dtype, nkv, hd, vd)
+    _need(nh % nkv == 0, lambda: f"{nh} heads do not divide into {nkv} key/value heads")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "block_tables must be contiguous int32 [requests, pages]")
+    for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
+        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), lambda: f"{name} must be int32 [tokens]")
+    out = torch.empty((T, nh, vd), dtype=q.dtype, device=q.device)
+    _run("paged_attention_general", library().ts_paged_attention_general(
+        _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
+        T, nh, nkv, hd, vd, k_cache.shape[1], *k_cache.stride()[:3], *v_cache.stride(), block_tables.shape[1],
+        float(scale), float(softcap), int(sink), int(window), _code(q.dtype), _page_run(pages_per_entry), _stream()))
+    return out
+
+
+def attention_general(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int, scale: float, *,
+                      softcap: float = 0.0, sink: bool = False, window: int = 0) -> torch.Tensor:
+    """Attention of a packed step over the cache for mixers with capped scores, a sink or values of
+    their own size; picks the kernel for the storage type and shape."""
+    tables = ctx.block_tables[space]
+    table_page = getattr(ctx, "page_size", 0) or k_cache.shape[1]
+    _need(table_page % k_cache.shape[1] == 0, lambda: f"block tables in pages of {table_page} over a cache in pages of {k_cache.shape[1]}")
+    per_entry = table_page // k_cache.shape[1]
+    return paged_attention_general(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, softcap=softcap,
+                                   sink=sink, window=window, pages_per_entry=per_entry)

@@ -119,3 +119,75 @@ class Attention(Mixer):
         if not isinstance(o, hip.SplitAttention):
             o = o.view(ctx.num_tokens, self.q_size)
         return linear(o, self.o, packed=self.o_packed, then=then)
+
+
+@register("mixer", "attention_general")
+class GeneralAttention(Mixer):
+    """Grouped-query attention with the options the fused rotate-half path above does not have, each
+    a constructor argument: value heads of a size of their own (`value_dim`), rotary positions taken
+    from frequencies (`position` names a `rotary_frequencies` encoding: interleaved or half pairs, a
+    leading part of the head), q and k heads divided by their root mean square after the rotation
+    (`qk_norm_eps`), value heads likewise before they are cached (`v_norm_eps`), scores capped as
+    softcap * tanh(score / softcap), and a softmax with a sink (one more in the denominator).
+    Separate q, k, v weights of a checkpoint land in row slices of one fused projection, whose output,
+    like the output projection's, is 32-bit; rotation, norms, scores and weights are 32-bit in every
+    storage type (`hip.qkv_finish`, `hip.paged_attention_general`)."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int | None = None,
+                 position: str | None = None, scale: float | None = None, softcap: float = 0.0, sink: bool = False,
+                 qk_norm_eps: float | None = None, v_norm_eps: float | None = None, window: int = 0) -> None:
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads do not divide into {num_kv_heads} key/value heads")
+        value_dim = head_dim if value_dim is None else value_dim
+        if not (0 < head_dim <= 256 and 0 < value_dim <= 256):
+            raise ValueError(f"head sizes {head_dim} / {value_dim}: the attention kernels take up to 256")
+        if softcap < 0:
+            raise ValueError(f"softcap {softcap}: positive, or 0 for none")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.value_dim, self.position = head_dim, value_dim, position
+        self.scale = scale if scale is not None else head_dim ** -0.5
+        self.softcap, self.sink, self.qk_norm_eps, self.v_norm_eps, self.window = softcap, sink, qk_norm_eps, v_norm_eps, window
+        self.qkv: torch.Tensor | None = None
+        self.o: torch.Tensor | None = None
+        self.qkv_packed: hip.StreamingCopies | None = None
+        self.o_packed: hip.StreamingCopies | None = None
+
+    @property
+    def q_size(self) -> int:
+        return self.num_heads * self.head_dim
+
+    @property
+    def k_size(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    @property
+    def v_size(self) -> int:
+        return self.num_kv_heads * self.value_dim
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {"qkv": ParamSpec((self.q_size + self.k_size + self.v_size, self.hidden_size)),
+                "o": ParamSpec((self.hidden_size, self.num_heads * self.value_dim))}
+
+    def kv_spec(self) -> KVSpec:
+        return KVSpec(self.num_kv_heads, self.head_dim, self.window,
+                      None if self.value_dim == self.head_dim else self.value_dim)
+
+    def keep_streaming_copies(self) -> int:
+        self.qkv_packed, self.o_packed = streaming_copy(self.qkv), streaming_copy(self.o)
+        return sum(c.nbytes() for c in (self.qkv_packed, self.o_packed) if c is not None)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
+        enc = ctx.position_encodings[self.position] if self.position else None
+        slots = ctx.slot_mapping[mem.space] if mem.store else None
+        k_store, v_store = (mem.k_cache, mem.v_cache) if mem.store else (None, None)
+        qkv = linear(x, self.qkv, out_dtype=torch.float32, packed=self.qkv_packed)
+        q = hip.qkv_finish(qkv, enc.frequencies() if enc is not None else None, ctx.positions, slots, k_store, v_store,
+                           self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, x.dtype,
+                           interleaved=getattr(enc, "interleaved", True), qk_norm_eps=self.qk_norm_eps,
+                           v_norm_eps=self.v_norm_eps)
+        o = hip.attention_general(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, softcap=self.softcap,
+                                  sink=self.sink, window=self.window)
+        return linear(o.view(ctx.num_tokens, self.num_heads * self.value_dim), self.o, out_dtype=torch.float32,
+                      packed=self.o_packed)

@@ -36,11 +36,17 @@ class ParamSpec:
 @dataclass(frozen=True)
 class KVSpec:
     """A mixer that caches a key and a value row per token. `window` 0 = every key is kept;
-    W > 0 = only the last W positions are ever read, so older pages can be given back."""
+    W > 0 = only the last W positions are ever read, so older pages can be given back.
+    `value_dim`: the size of a head's value row where it differs from its key row's (None: `head_dim`)."""
 
     num_kv_heads: int
     head_dim: int
     window: int = 0
+    value_dim: int | None = None
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)
@@ -154,6 +160,10 @@ class PositionEncoding(Part):
 
     def rotary_table(self) -> torch.Tensor | None:
         """float32 [positions, head_dim] = [cos | sin] for rotate-half mixers, or None."""
+        return None
+
+    def frequencies(self) -> torch.Tensor | None:
+        """float64 [rotary_dim / 2] for mixers whose kernels take the angles themselves, or None."""
         return None
 
     def on_embedding(self, hidden: torch.Tensor, ctx: StepContext) -> torch.Tensor:

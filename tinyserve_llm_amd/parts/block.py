@@ -13,7 +13,7 @@ that norm, deferred, as its `hidden` (with `residual` None: the sum is inside)."
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
 import torch
 
@@ -26,6 +26,7 @@ class Layer:
     feed_forward: FeedForward
     norms: dict[str, Norm]           # by the names the arrangement uses
     block: str = "pre_norm"
+    block_args: dict = field(default_factory=dict)      # the arrangement's own constants (a residual multiplier, say)
 
     def parts(self) -> dict[str, object]:
         """Every part by the name its parameters are known under (`layers.<i>.<name>.<parameter>`)."""
@@ -97,3 +98,35 @@ def pre_norm_block(layer: Layer, hidden, residual: torch.Tensor | None, ctx: Ste
     if following is not None and following.made_for(x):
         residual = None
     return x, residual
+
+
+def keeps_stream(fn):
+    """Declares that an arrangement takes a `parts.stream.ResidualStream` as `hidden` (with `residual`
+    None) and returns one: a model whose residual stream is 32-bit is made of such arrangements."""
+    fn.keeps_stream = True
+    return fn
+
+
+@register("block", "parallel")
+@uses_norms("norm1", "norm2")
+@keeps_stream
+def parallel_block(layer: Layer, hidden, residual, ctx: StepContext, mem: LayerMemory):
+    """x <- x + mult * (mixer(norm1(x)) + feed_forward(norm2(x))): both branches read the same x, each
+    through a norm of its own; `mult` is the layer's `block_args["residual_mult"]` (1 if not given). The
+    stream is 32-bit. The sum is left pending in the stream that comes back, so that the next layer's
+    two norms (or the final norm) are made by the kernel that adds it; the two norms of a layer share
+    one mean square."""
+    from tinyserve_llm_amd.parts.stream import ResidualStream
+    if not isinstance(hidden, ResidualStream) or residual is not None:
+        raise TypeError("the parallel arrangement runs on a 32-bit residual stream (ModelSpec.residual_dtype = 'float32')")
+    norm1, norm2 = layer.norms["norm1"], layer.norms["norm2"]
+    if norm1.eps != norm2.eps:
+        raise ValueError("the two norms of a parallel layer share their mean square, so also their eps")
+    x, h1, h2 = hidden.settle((norm1.weight, norm2.weight), norm1.eps, norm1.weight.dtype)
+    a = layer.mixer.forward(h1, ctx, mem)
+    ff = layer.feed_forward
+    if getattr(ff, "can_defer_bias", False):
+        b, bias = ff.forward(h2, ctx, defer_bias=True)
+    else:
+        b, bias = ff.forward(h2, ctx), None
+    return ResidualStream(x, a, b, bias, float(layer.block_args.get("residual_mult", 1.0))), None

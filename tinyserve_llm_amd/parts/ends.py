@@ -11,14 +11,19 @@ import torch
 from tinyserve_llm_amd.ops import hip
 from tinyserve_llm_amd.parts.base import Embedding, Head, ParamSpec, StepContext, register
 from tinyserve_llm_amd.parts.linear import linear, streaming_copy
+from tinyserve_llm_amd.parts.stream import ResidualStream
 
 
 @register("embedding", "table")
 class TableEmbedding(Embedding):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, init: tuple[float, float] = (0.0, 0.02)) -> None:
+    def __init__(self, vocab_size: int, hidden_size: int, init: tuple[float, float] = (0.0, 0.02),
+                 float32_stream: bool = False) -> None:
+        """`float32_stream`: the rows start a residual stream that is kept in 32-bit floats
+        (`parts.stream.ResidualStream`) whatever the table's storage type."""
         self.vocab_size, self.hidden_size, self.init = vocab_size, hidden_size, tuple(init)
+        self.float32_stream = float32_stream
         self.weight: torch.Tensor | None = None
 
     def param_specs(self) -> dict[str, ParamSpec]:
@@ -27,7 +32,9 @@ class TableEmbedding(Embedding):
     def table(self) -> torch.Tensor | None:
         return self.weight
 
-    def forward(self, ctx: StepContext) -> torch.Tensor:
+    def forward(self, ctx: StepContext) -> "torch.Tensor | ResidualStream":
+        if self.float32_stream:
+            return ResidualStream(hip.embedding_stream(self.weight, ctx.token_ids))
         return hip.embedding(self.weight, ctx.token_ids)      # (ids are checked against the vocabulary on the host)
 
 

@@ -5,6 +5,7 @@ from __future__ import annotations
 
 import torch
 
+from tinyserve_llm_amd.ops import hip
 from tinyserve_llm_amd.parts.base import FeedForward, ParamSpec, StepContext, register
 from tinyserve_llm_amd.parts.linear import linear, streaming_copy
 
@@ -36,3 +37,55 @@ class GatedMLP(FeedForward):
     def forward(self, x: torch.Tensor, ctx: StepContext, then=None) -> torch.Tensor:
         gated = linear(x, self.gate_up, glu=True, packed=self.gate_up_packed, feeds=self.down)
         return linear(gated, self.down, packed=self.down_packed, then=then)
+
+
+@register("feed_forward", "dense_mlp")
+class DenseMLP(FeedForward):
+    """A feed-forward without a gate: W_down act(W_up h + b_up) + b_down, `activation` one of
+    `hip.ACTIVATIONS` ("relu2": the square of relu). The up projection's sums stay 32-bit until bias and
+    activation are applied; the down projection's result is 32-bit. `forward(..., defer_bias=True)`
+    returns (W_down a, b_down) for a caller that adds the bias with its residual sum."""
+
+    graph_safe = True
+    can_defer_bias = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu2", bias: bool = True) -> None:
+        if activation not in hip.ACTIVATIONS:
+            raise ValueError(f"activation {activation!r}: one of {sorted(hip.ACTIVATIONS)}")
+        self.hidden_size, self.intermediate_size, self.activation, self.has_bias = hidden_size, intermediate_size, activation, bias
+        self.up: torch.Tensor | None = None
+        self.down: torch.Tensor | None = None
+        self.up_bias: torch.Tensor | None = None
+        self.down_bias: torch.Tensor | None = None
+        self.up_packed = None
+        self.down_packed = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        specs = {"up": ParamSpec((self.intermediate_size, self.hidden_size)),
+                 "down": ParamSpec((self.hidden_size, self.intermediate_size))}
+        if self.has_bias:
+            specs["up_bias"] = ParamSpec((self.intermediate_size,), init=(0.0, 0.1))
+            specs["down_bias"] = ParamSpec((self.hidden_size,), init=(0.0, 0.1))
+        return specs
+
+    def keep_streaming_copies(self) -> int:
+        self.up_packed, self.down_packed = streaming_copy(self.up), streaming_copy(self.down)
+        return sum(c.nbytes() for c in (self.up_packed, self.down_packed) if c is not None)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, defer_bias: bool = False):
+        up = linear(x, self.up, out_dtype=torch.float32, packed=self.up_packed)
+        act = hip.bias_activation(up, self.up_bias, self.activation, x.dtype)
+        down = linear(act, self.down, out_dtype=torch.float32, packed=self.down_packed)
+        if defer_bias:
+            return down, self.down_bias
+        return down if self.down_bias is None else hip.bias_activation(down, self.down_bias, "none", torch.float32)
+
+
+@register("feed_forward", "none")
+class NoFeedForward(FeedForward):
+    """A layer without a feed-forward: `forward` gives None, which a block's residual sum leaves out."""
+
+    graph_safe = True
+
+    def forward(self, x, ctx: StepContext, **_):
+        return None

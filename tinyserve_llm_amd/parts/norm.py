@@ -12,6 +12,7 @@ import torch
 from tinyserve_llm_amd.ops import hip
 from tinyserve_llm_amd.parts.base import Norm, ParamSpec, register
 from tinyserve_llm_amd.parts.linear import DeferredNorm, NormRequest
+from tinyserve_llm_amd.parts.stream import ResidualStream
 
 
 @register("norm", "rmsnorm")
@@ -27,6 +28,11 @@ class RMSNorm(Norm):
         return {"weight": ParamSpec((self.hidden_size,), init=(1.0, 0.1))}
 
     def __call__(self, x, residual=None, rows=None):
+        if isinstance(x, ResidualStream):
+            # a 32-bit stream: its pending sum, then the norm, rounded to the weights' storage type on the way out
+            if residual is not None:
+                raise ValueError("a residual stream carries its own sum")
+            return x.norm_rows(rows, self.weight, self.eps, self.weight.dtype), (None if rows is not None else x.x)
         return hip.rmsnorm(x, self.weight, self.eps, residual, rows)
 
     def defer(self, x, residual=None) -> DeferredNorm:

@@ -59,3 +59,30 @@ class Rope(PositionEncoding):
 
     def rotary_table(self) -> torch.Tensor | None:
         return self.cos_sin
+
+
+@register("position_encoding", "rotary_frequencies")
+class RotaryFrequencies(PositionEncoding):
+    """Rotary positions without a table over positions, for models that set no limit to a request's
+    length: only the frequencies f_i = theta^(-2i / rotary_dim), i < rotary_dim / 2, are kept (64-bit),
+    and a mixer's kernel takes the angle position * f_i itself. `interleaved`: pair i is dimensions
+    (2i, 2i+1) of a head; otherwise (i, i + rotary_dim/2). The first `rotary_dim` dimensions of a head
+    turn, the rest pass."""
+
+    graph_safe = True
+
+    def __init__(self, rotary_dim: int, theta: float, interleaved: bool = True) -> None:
+        if rotary_dim % 2 or rotary_dim < 0:
+            raise ValueError(f"rotary_dim {rotary_dim}: an even number of dimensions turns")
+        self.rotary_dim, self.theta, self.interleaved = rotary_dim, float(theta), interleaved
+        self.freqs: torch.Tensor | None = None
+
+    def host_frequencies(self) -> torch.Tensor:
+        i = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
+        return torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / max(1, self.rotary_dim))
+
+    def prepare(self, device: torch.device) -> None:
+        self.freqs = self.host_frequencies().to(device) if self.rotary_dim else None
+
+    def frequencies(self) -> torch.Tensor | None:
+        return self.freqs
