@@ -39,3 +39,21 @@ def make_folder(tmp_path_factory, name: str) -> str:
 def prompt(seed: int, length: int, vocab: int) -> list[int]:
     rng = random.Random(seed)
     return [rng.randrange(vocab) for _ in range(length)]
+
+
+def rugezen_configs():
+    """Two small Rugezen configurations that differ from each other in every size and option: key/value
+    grouping, key and value head sizes (equal or not), how much of a head turns, caps, layer order, a
+    looped stretch (three passes over two layers, or none), a layer without feed-forward, eps, the
+    residual multiplier, and widths that are no multiples of 64."""
+    from tinyserve_llm_amd.config.rugezen import RugezenAttention, RugezenConfig, RugezenLayer, RugezenMinGRU
+    att_p = RugezenAttention(heads=4, kv_heads=2, dim=32, vdim=48, rot_dims=16, rot_base=10000.0, scale=0.31, softcap=3.0)
+    att_q = RugezenAttention(heads=2, kv_heads=2, dim=16, vdim=16, rot_dims=16, rot_base=700.0, scale=0.25, softcap=30.0)
+    att_r = RugezenAttention(heads=6, kv_heads=1, dim=24, vdim=8, rot_dims=4, rot_base=50000.0, scale=0.2, softcap=1.5)
+    P = RugezenConfig(vocab=200, width=80, norm_eps=1e-6, residual_mult=0.37, loop_start=0, loop_stop=2, loop_times=3,
+                      layers=(RugezenLayer("mingru", RugezenMinGRU(width=72), 96), RugezenLayer("attention", att_p, 144),
+                              RugezenLayer("attention", att_r, None)))
+    Q = RugezenConfig(vocab=131, width=48, norm_eps=1e-4, residual_mult=1.0,
+                      layers=(RugezenLayer("attention", att_q, 64), RugezenLayer("mingru", RugezenMinGRU(width=100), None),
+                              RugezenLayer("mingru", RugezenMinGRU(width=16), 40), RugezenLayer("attention", att_p, 56)))
+    return {"P": (P, 3), "Q": (Q, 4)}

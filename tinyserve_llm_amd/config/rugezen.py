@@ -37,7 +37,7 @@ class RugezenAttention:
                 rot_dims=int(_need(rot, "dims", where + ".rot")), rot_base=float(_need(rot, "base", where + ".rot")),
                 scale=float(_need(raw, "scale", where)), softcap=float(_need(raw, "softcap", where)))
         if c.heads <= 0 or c.kv_heads <= 0 or c.heads % c.kv_heads:
-            raise ConfigError(f"{where}: {c.heads} heads do not divide into {c.kv_heads} key/value heads")
+            raise ConfigError(f"{where}.kv_heads: {c.heads} heads do not divide into {c.kv_heads} key/value heads")
         if c.rot_dims % 2 or not 0 <= c.rot_dims <= c.dim:
             raise ConfigError(f"{where}.rot.dims {c.rot_dims}: an even number up to dim {c.dim}")
         if c.softcap <= 0:

@@ -21,12 +21,12 @@ def rugezen_spec(config: RugezenConfig) -> ModelSpec:
     norm = PartSpec("rmsnorm", dict(hidden_size=c.width, eps=c.norm_eps))
     layers: list[LayerSpec] = []
     encodings: dict[str, PartSpec] = {}
+    unused: list[str] = []
     ckpt: dict[str, Destination] = {"embed": Destination("embed.weight"), "final.norm": Destination("final_norm.weight"),
                                     "head": Destination("head.weight")}
     for i, layer in enumerate(c.layers):
         src, dst = f"l{i}", f"layers.{i}"
         ckpt[f"{src}.norm1"] = Destination(f"{dst}.norm1.weight")
-        ckpt[f"{src}.norm2"] = Destination(f"{dst}.norm2.weight")
         m = layer.mixer
         if isinstance(m, RugezenAttention):
             # one encoding per distinct (dims, base): layers that turn alike share its frequencies
@@ -51,19 +51,23 @@ def rugezen_spec(config: RugezenConfig) -> ModelSpec:
             ckpt[f"{src}.mix.z.b"] = Destination(f"{dst}.mixer.bias", 0, w)
             ckpt[f"{src}.mix.x.b"] = Destination(f"{dst}.mixer.bias", w, w)
             ckpt[f"{src}.mix.o"] = Destination(f"{dst}.mixer.o")
+        norms = {"norm1": norm}
         if layer.ff is None:
             ff = PartSpec("none")
+            unused.append(f"{src}.norm2")        # (a checkpoint may carry the norm of the branch that is not there)
         else:
+            norms["norm2"] = norm
+            ckpt[f"{src}.norm2"] = Destination(f"{dst}.norm2.weight")
             ff = PartSpec("dense_mlp", dict(hidden_size=c.width, intermediate_size=layer.ff, activation="relu2", bias=True))
             ckpt[f"{src}.mlp.up"] = Destination(f"{dst}.ff.up")
             ckpt[f"{src}.mlp.up.b"] = Destination(f"{dst}.ff.up_bias")
             ckpt[f"{src}.mlp.down"] = Destination(f"{dst}.ff.down")
             ckpt[f"{src}.mlp.down.b"] = Destination(f"{dst}.ff.down_bias")
-        layers.append(LayerSpec(mixer, ff, {"norm1": norm, "norm2": norm}, "parallel", {"residual_mult": c.residual_mult}))
+        layers.append(LayerSpec(mixer, ff, norms, "parallel", {"residual_mult": c.residual_mult}))
     return ModelSpec(
         architecture=c.architecture, vocab_size=c.vocab, hidden_size=c.width, max_position=None, layers=layers,
         order=[LayerRun(i) for i in c.run_order()], final_norm=norm, position_encodings=encodings,
-        tie_word_embeddings=False, residual_dtype="float32", checkpoint=ckpt)
+        tie_word_embeddings=False, residual_dtype="float32", checkpoint=ckpt, optional=tuple(unused))
 
 
 RUGEZEN = register_architecture(Architecture(

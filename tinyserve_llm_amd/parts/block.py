@@ -108,24 +108,26 @@ def keeps_stream(fn):
 
 
 @register("block", "parallel")
-@uses_norms("norm1", "norm2")
+@uses_norms("norm1")
 @keeps_stream
 def parallel_block(layer: Layer, hidden, residual, ctx: StepContext, mem: LayerMemory):
     """x <- x + mult * (mixer(norm1(x)) + feed_forward(norm2(x))): both branches read the same x, each
-    through a norm of its own; `mult` is the layer's `block_args["residual_mult"]` (1 if not given). The
-    stream is 32-bit. The sum is left pending in the stream that comes back, so that the next layer's
+    through a norm of its own ("norm1", "norm2"; a layer whose feed-forward is "none" needs no
+    "norm2"); `mult` is the layer's `block_args["residual_mult"]` (1 if not given). The stream is 32-bit. The sum is left pending in the stream that comes back, so that the next layer's
     two norms (or the final norm) are made by the kernel that adds it; the two norms of a layer share
     one mean square."""
     from tinyserve_llm_amd.parts.stream import ResidualStream
     if not isinstance(hidden, ResidualStream) or residual is not None:
         raise TypeError("the parallel arrangement runs on a 32-bit residual stream (ModelSpec.residual_dtype = 'float32')")
-    norm1, norm2 = layer.norms["norm1"], layer.norms["norm2"]
-    if norm1.eps != norm2.eps:
+    norm1, norm2 = layer.norms["norm1"], layer.norms.get("norm2")
+    if norm2 is not None and norm1.eps != norm2.eps:
         raise ValueError("the two norms of a parallel layer share their mean square, so also their eps")
-    x, h1, h2 = hidden.settle((norm1.weight, norm2.weight), norm1.eps, norm1.weight.dtype)
+    x, h1, h2 = hidden.settle((norm1.weight, None if norm2 is None else norm2.weight), norm1.eps, norm1.weight.dtype)
     a = layer.mixer.forward(h1, ctx, mem)
     ff = layer.feed_forward
-    if getattr(ff, "can_defer_bias", False):
+    if norm2 is None:
+        b, bias = ff.forward(None, ctx), None          # (only a part that reads nothing can do without its norm)
+    elif getattr(ff, "can_defer_bias", False):
         b, bias = ff.forward(h2, ctx, defer_bias=True)
     else:
         b, bias = ff.forward(h2, ctx), None
