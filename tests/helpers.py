@@ -50,10 +50,11 @@ def rugezen_configs():
     att_p = RugezenAttention(heads=4, kv_heads=2, dim=32, vdim=48, rot_dims=16, rot_base=10000.0, scale=0.31, softcap=3.0)
     att_q = RugezenAttention(heads=2, kv_heads=2, dim=16, vdim=16, rot_dims=16, rot_base=700.0, scale=0.25, softcap=30.0)
     att_r = RugezenAttention(heads=6, kv_heads=1, dim=24, vdim=8, rot_dims=4, rot_base=50000.0, scale=0.2, softcap=1.5)
+    att_s = RugezenAttention(heads=4, kv_heads=2, dim=64, vdim=64, rot_dims=32, rot_base=1000.0, scale=0.15, softcap=2.5)
     P = RugezenConfig(vocab=200, width=80, norm_eps=1e-6, residual_mult=0.37, loop_start=0, loop_stop=2, loop_times=3,
                       layers=(RugezenLayer("mingru", RugezenMinGRU(width=72), 96), RugezenLayer("attention", att_p, 144),
                               RugezenLayer("attention", att_r, None)))
     Q = RugezenConfig(vocab=131, width=48, norm_eps=1e-4, residual_mult=1.0,
                       layers=(RugezenLayer("attention", att_q, 64), RugezenLayer("mingru", RugezenMinGRU(width=100), None),
-                              RugezenLayer("mingru", RugezenMinGRU(width=16), 40), RugezenLayer("attention", att_p, 56)))
+                              RugezenLayer("mingru", RugezenMinGRU(width=16), 40), RugezenLayer("attention", att_s, 56)))
     return {"P": (P, 3), "Q": (Q, 4)}

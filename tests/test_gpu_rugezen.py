@@ -238,6 +238,71 @@ def test_attention_far_keys_page_borders_and_first_tokens(dtype, sizes):
         torch.testing.assert_close(out, want, **tol)
 
 
+def step_context(table, page, starts, counts):
+    """A packed step over requests that all read the pages `table` names: request i feeds `counts[i]`
+    tokens from position `starts[i]`."""
+    from tinyserve_llm_amd.parts.base import StepContext
+    positions, seq_of, cu = [], [], [0]
+    for i, (s0, n) in enumerate(zip(starts, counts)):
+        positions += list(range(s0, s0 + n))
+        seq_of += [i] * n
+        cu.append(cu[-1] + n)
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    ends = [a + b for a, b in zip(starts, counts)]
+    return StepContext(num_tokens=len(positions), num_seqs=len(starts), token_ids=dev([0] * len(positions)), positions=dev(positions),
+                       seq_of_token=dev(seq_of), cu_seqlens=dev(cu), context_lens=dev(ends), state_slots=dev([0] * len(starts)),
+                       slot_mapping=[], block_tables=[table.view(1, -1).repeat(len(starts), 1).contiguous().to(DEV)],
+                       host_cu_seqlens=cu, host_starts=list(starts), host_context_lens=ends, host_state_slots=[0] * len(starts),
+                       page_size=page), positions
+
+
+@pytest.mark.parametrize("sizes", [(4, 1, 96, 96), (8, 2, 64, 64), (2, 2, 128, 128), (4, 4, 32, 32), (16, 1, 64, 64)])
+@pytest.mark.parametrize("cap, sink", [(30.0, True), (0.0, True), (0.8, False)])
+def test_matrix_core_kernels_general_variants(sizes, cap, sink):
+    """bfloat16 heads of the matrix-core kernels' sizes go to those kernels' general variants: single
+    tokens (whole walks and walks cut into chunks), a long portion, and single tokens leading a portion
+    in one step; far keys, keys at both sides of page borders and of the 32-key steps, the first tokens."""
+    h = hip()
+    H, G, D, V = sizes
+    page, length = 32, 2300
+    stand_out = {2299: 3, 2250: 31, 2251: 32, 2252: 33, 2253: 2253, 2200: 63, 2201: 64, 2100: 1023, 2101: 1024, 40: 0, 2222: 2221}
+    gen = torch.Generator().manual_seed(5)
+    k64 = plain.unit_rms(torch.randn(length, G, D, generator=gen, dtype=F64), 0.0)
+    v64 = torch.randn(length, G, V, generator=gen, dtype=F64)
+    q64 = plain.unit_rms(torch.randn(length, H, D, generator=gen, dtype=F64), 0.0)
+    for p, key in stand_out.items():
+        g_dir = plain.unit_rms(torch.randn(G, D, generator=gen, dtype=F64), 0.0)
+        for hh in range(H):
+            q64[p, hh] = g_dir[hh // (H // G)]
+        k64[key] = 3 * g_dir
+    pages = -(-length // page)
+    table = torch.randperm(pages + 5, generator=gen)[:pages].to(torch.int32)
+    k, v = paged(pages + 5, page, G, D, V, torch.bfloat16)
+    kr, vr = k64.to(torch.bfloat16), v64.to(torch.bfloat16)
+    idx = (table.long()[torch.arange(length) // page], torch.arange(length) % page)
+    k[idx[0].to(DEV), idx[1].to(DEV)] = kr.to(DEV)
+    v[idx[0].to(DEV), idx[1].to(DEV)] = vr.to(DEV)
+    qr = q64.to(torch.bfloat16)
+    scale = D ** -0.5
+    tol = dict(atol=2e-2, rtol=2e-2)
+
+    def run(starts, counts):
+        ctx, positions = step_context(table, page, starts, counts)
+        q = qr[positions].to(DEV).contiguous()
+        assert h.decode_kernel_takes(q, k, v), "these sizes are the matrix-core kernels'"
+        out = h.paged_attention(q, k, v, ctx, 0, scale, 0, softcap=cap, sink=sink)
+        want = plain.sink_attention(qr[positions].to(F64), kr.to(F64), vr.to(F64), torch.tensor(positions), scale, cap, sink)
+        torch.testing.assert_close(out.cpu().to(F64), want, msg=lambda m: f"starts {starts} counts {counts}: {m}", **tol)
+
+    for pos in (0, 1, 31, 32, 40, 2100, 2101, 2299):
+        run([pos], [1])                                   # one token, one request
+    run([2299, 40, 2250, 0, 2201, 2222, 33, 2100], [1] * 8)   # a batch of single tokens of unequal contexts
+    run([2180], [120])                                    # a portion deep in a request
+    run([0], [70])                                        # the first tokens as a portion
+    run([2252, 2253, 2190], [1, 1, 110])                  # single tokens lead a portion
+    run([2296], [2])                                      # a portion of two tokens
+
+
 def test_the_sink_weighs_most_on_the_first_tokens():
     """One visible key of score s: the weight is e^s / (1 + e^s), not 1."""
     out, want, v = attention_case(torch.float32, 2, 1, 16, 16, 16, 3, [0], {}, 0.25, 50.0, True)

@@ -23,17 +23,19 @@
 
 // ONE: a wave has a single 32-key step (chunk = 32 waves); without the second buffer of the
 // general loop the kernel needs fewer registers and more workgroups share a compute unit
-template <int HD, bool ONE>
+// GENERAL: capped scores, weights in two terms (attention_mfma.h), and optionally a sink: one more in the
+// softmax's denominator, added where a token's chunks meet (here with one chunk, else in the combining kernel).
+template <int HD, bool ONE, bool GENERAL>
 __global__ void __launch_bounds__(DEC_WAVES_FOR(HD, ONE) * TS_WAVE)
 attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
                         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                         const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
                         const int32_t* __restrict__ positions, int nh, int G, int page_size, int page_shift, int page_run,
                         int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
-                        int num_splits, int chunk, float scale2, int window) {
+                        int num_splits, int chunk, float scale2, int window, float cap_in, float cap_out, int sink) {
   constexpr int NC = HD / 32;    // 32-dimension pieces of a key row (one 16-byte load per lane each)
   constexpr int NDB = HD / 16;   // 16-dimension blocks of the output
-  ts_fetch_arguments<164>();     // (nine pointers, five numbers, six strides, four more numbers and the scale)
+  ts_fetch_arguments<GENERAL ? 176 : 164>();     // (nine pointers, five numbers, six strides, four more numbers and the scale; the caps and the sink)
   extern __shared__ __align__(16) float smem[];
   const int nw = blockDim.x / TS_WAVE;
   float* wm = smem;                       // [waves][16]
@@ -73,7 +75,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
   if (kend > pos + 1) kend = pos + 1;
   int kb = (k0 > (lo & ~31) ? k0 : (lo & ~31)) + 32 * wave;
 #define TS_LOAD(T, KB) load_tile<HD>(T, KB, r, g, lo, pos, kvh, table, pm, k_cache, v_cache, kp, ks, kh, vp, vh, vd)
-#define TS_USE(T, KB) use_tile_auto<HD>(T, KB, r, g, lo, pos, pos, lo, qreg, scale2, m, l, o)
+#define TS_USE(T, KB) use_tile_auto<HD, GENERAL>(T, KB, r, g, lo, pos, pos, lo, qreg, scale2, m, l, o, cap_in, cap_out)
   if (ONE) {
     if (kb < kend) {
       KVTile<HD> A;
@@ -123,6 +125,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
       L = fmaf(wl[w * 16 + head], wgt, L);
     }
     if (num_splits == 1) {                  // the whole context was this workgroup's: position `pos` is always visible
+      if (GENERAL && sink) L += fast_exp2(-M);
       out[((int64_t)t * nh + (int64_t)kvh * G + head) * HD + d] = f2bf(acc / L);
     } else {
       const int64_t row = ((int64_t)t * nh + (int64_t)kvh * G + head) * num_splits + split;
@@ -140,7 +143,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
 __global__ void __launch_bounds__(TS_WAVE)
 attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                            const float* __restrict__ part_ml, const int32_t* __restrict__ positions, int nh, int hd,
-                           int num_splits, int chunk, int window) {
+                           int num_splits, int chunk, int window, int sink) {
   __shared__ float wgt[COMBINE_MAX_SPLITS];
   const int t = blockIdx.x / nh, lane = threadIdx.x;
   const int64_t th = blockIdx.x;
@@ -158,6 +161,7 @@ attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ p
     L += ml[2 * s + 1] * w;
   }
   L = wave_sum(L);
+  if (sink) L += fast_exp2(-M);           // the sink's score is 0
   wave_sync();
   const float inv = 1.0f / L;
   const float* po = part_o + (th * num_splits + s0) * hd;
@@ -181,10 +185,10 @@ extern "C" int ts_attention_combine(void* out, const float* part_o, const float*
 // The combining kernel alone, for the prefill kernel's split walks (declared in attention_mfma.h).
 int ts_launch_attention_combine(void* out, const float* part_o, const float* part_ml, const int32_t* positions,
                                 int num_tokens, int nh, int hd, int num_splits, int chunk, int window,
-                                hipStream_t stream) {
+                                hipStream_t stream, int sink) {
   if (num_splits > COMBINE_MAX_SPLITS) return TS_BAD_SHAPE;
   attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,
-                                                                      num_splits, chunk, window);
+                                                                      num_splits, chunk, window, sink);
   return ts_check_launch();
 }
 
@@ -196,12 +200,13 @@ int ts_launch_attention_combine(void* out, const float* part_o, const float* par
 // head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages, slot stride 1, strides
 // vp/vh/vd (page, head, dimension). An entry of block_tables names 2^page_run consecutive pages of page_size
 // keys (entry e: the pages e 2^page_run + j); max_blocks is the tables' width in entries.
-extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_ml, const void* q, const void* k_cache,
-                                         const void* v_cache, const int32_t* block_tables,
-                                         const int32_t* seq_of_token, const int32_t* positions, int num_tokens, int nh,
-                                         int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
-                                         int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits, int chunk,
-                                         int waves, float scale, int window, int page_run, int combine, hipStream_t stream) {
+static int launch_decode(void* out, float* part_o, float* part_ml, const void* q, const void* k_cache,
+                         const void* v_cache, const int32_t* block_tables,
+                         const int32_t* seq_of_token, const int32_t* positions, int num_tokens, int nh,
+                         int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
+                         int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits, int chunk,
+                         int waves, float scale, int window, int page_run, int combine, bool general, float softcap, int sink,
+                         hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || num_splits <= 0 || page_run < 0 || page_run > 16)
     return TS_BAD_SHAPE;
@@ -222,12 +227,17 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
     while ((1 << page_shift) < page_size) ++page_shift;
   }
   dim3 grid(num_splits, nkv, num_tokens);
-#define TS_DEC1(HH, ON)                                                                                         \
-  attn_decode_mfma_kernel<HH, ON><<<grid, waves * TS_WAVE, smem, stream>>>(                                 \
+  // capped: the cap's tanh takes the scale in and gives units of log2 out, and the softmax's own scale is 1
+  const float log2e = 1.44269504088896340736f;
+  const float cap_in = softcap > 0.f ? scale / softcap : 0.f, cap_out = softcap * log2e;
+  const float scale2 = softcap > 0.f ? 1.0f : scale * log2e;
+#define TS_DEC2(HH, ON, GG)                                                                                     \
+  attn_decode_mfma_kernel<HH, ON, GG><<<grid, waves * TS_WAVE, smem, stream>>>(                                 \
       (bf16_t*)out, part_o, part_ml, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,          \
       block_tables, seq_of_token, positions, nh, G, page_size, page_shift, page_run, kp, ks, kh, vp, vh, vd, max_blocks,  \
-      num_splits, chunk, scale * 1.44269504088896340736f, window)
-#define TS_DEC(HH) if (chunk == 32 * waves) TS_DEC1(HH, true); else TS_DEC1(HH, false)
+      num_splits, chunk, scale2, window, cap_in, cap_out, sink)
+#define TS_DEC1(HH, ON) if (general) TS_DEC2(HH, ON, true); else TS_DEC2(HH, ON, false)
+#define TS_DEC(HH) if (chunk == 32 * waves) { TS_DEC1(HH, true); } else { TS_DEC1(HH, false); }
   switch (hd) {
     case 32: TS_DEC(32); break;
     case 64: TS_DEC(64); break;
@@ -237,9 +247,36 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
   }
 #undef TS_DEC
 #undef TS_DEC1
+#undef TS_DEC2
   int rc = ts_check_launch();
   if (rc || num_splits == 1 || !combine) return rc;     // (combine 0: the caller's next kernel reads the parts itself)
   attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,
-                                                                      num_splits, chunk, window);
+                                                                      num_splits, chunk, window, general ? sink : 0);
   return ts_check_launch();
+}
+
+extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_ml, const void* q, const void* k_cache,
+                                         const void* v_cache, const int32_t* block_tables,
+                                         const int32_t* seq_of_token, const int32_t* positions, int num_tokens, int nh,
+                                         int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
+                                         int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits, int chunk,
+                                         int waves, float scale, int window, int page_run, int combine, hipStream_t stream) {
+  return launch_decode(out, part_o, part_ml, q, k_cache, v_cache, block_tables, seq_of_token, positions, num_tokens, nh, nkv, hd,
+                       page_size, kp, ks, kh, vp, vh, vd, max_blocks, num_splits, chunk, waves, scale, window, page_run, combine,
+                       false, 0.f, 0, stream);
+}
+
+// The same with capped scores (softcap > 0: cap * tanh(score / cap)), a sink (one more in the softmax's
+// denominator) and weights carried in two bfloat16 terms; always combines.
+extern "C" int ts_paged_attention_decode_general(void* out, float* part_o, float* part_ml, const void* q, const void* k_cache,
+                                                 const void* v_cache, const int32_t* block_tables,
+                                                 const int32_t* seq_of_token, const int32_t* positions, int num_tokens,
+                                                 int nh, int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
+                                                 int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits,
+                                                 int chunk, int waves, float scale, int window, int page_run, float softcap,
+                                                 int sink, hipStream_t stream) {
+  if (softcap < 0.f) return TS_BAD_SHAPE;
+  return launch_decode(out, part_o, part_ml, q, k_cache, v_cache, block_tables, seq_of_token, positions, num_tokens, nh, nkv, hd,
+                       page_size, kp, ks, kh, vp, vh, vd, max_blocks, num_splits, chunk, waves, scale, window, page_run, 1,
+                       true, softcap, sink, stream);
 }

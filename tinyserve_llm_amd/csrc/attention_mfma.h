@@ -141,12 +141,28 @@ static __device__ __forceinline__ void tile_scores(const uint4 (&k)[2][HD / 32],
 // MASKED: rows mask the keys beyond their position and before their window (`vok`: whether any of
 // this lane's eight keys of v is visible); without it every key of the step is visible to every row
 // (the caller has checked).
-template <int HD, bool MASKED, typename L>
+// GENERAL: the variant for mixers with capped scores and weights that must not lose their 32 bits. With cap_in
+// != 0 a score becomes cap_out * tanh(score * cap_in) first (cap_in = scale / cap, cap_out = cap * log2 e, and
+// scale2 = 1); and the weights enter the products as two bfloat16 terms, P = hi + lo with lo = P - hi rounded
+// again, which carries 16 bits of their mantissa (the plain variant rounds P to 8).
+template <int HD, bool MASKED, typename L, bool GENERAL = false>
 static __device__ __forceinline__ void tile_softmax_values(float4_t (&s)[2], const uint4 (&v)[HD / 16], bool vok, int kb, int r,
                                                            int g, int lo, int pos, float scale2, float& m, L& l,
-                                                           float4_t (&o)[HD / 16]) {
+                                                           float4_t (&o)[HD / 16], float cap_in = 0.f, float cap_out = 0.f) {
   constexpr int NDB = HD / 16;
   constexpr bool SUMS_BY_MFMA = std::is_same<L, float4_t>::value;
+  if constexpr (GENERAL) {
+    if (cap_in != 0.f) {
+      // tanh(x) = 1 - 2 / (1 + e^(2x)), by the hardware's 2^x and reciprocal
+#pragma unroll
+      for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float e = fast_exp2(s[tau][j] * (cap_in * 2.88539008177792681472f));
+          s[tau][j] = cap_out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e));
+        }
+    }
+  }
   // this lane: row r, keys kb + 8 g + 4 tau + j
   float mloc = -INFINITY;
 #pragma unroll
@@ -196,31 +212,50 @@ static __device__ __forceinline__ void tile_softmax_values(float4_t (&s)[2], con
     const uint32_t ones = 0x3f803f80u;                 // 1.0 twice (a masked key's P is 0 already)
     l = mfma32(pa, make_uint4(ones, ones, ones, ones), l);
   }
+  if constexpr (GENERAL) {
+    // what the rounding of P left out, rounded again: the second term of the weights
+    const uint32_t hi[4] = {pa.x, pa.y, pa.z, pa.w};
+    uint32_t lo2[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float pe = p[w >> 1][2 * (w & 1)], po = p[w >> 1][2 * (w & 1) + 1];
+      lo2[w] = pack_bf16(pe - __uint_as_float(hi[w] << 16), po - __uint_as_float(hi[w] & 0xffff0000u));
+    }
+    const uint4 pb = make_uint4(lo2[0], lo2[1], lo2[2], lo2[3]);
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) o[db] = mfma32(pb, (MASKED && !vok) ? make_uint4(0, 0, 0, 0) : v[db], o[db]);
+    if constexpr (SUMS_BY_MFMA) {
+      const uint32_t ones = 0x3f803f80u;
+      l = mfma32(pb, make_uint4(ones, ones, ones, ones), l);
+    }
+  }
 }
 
 // One 32-key step whole: the scores, then the softmax and the values.
-template <int HD, bool MASKED, typename L>
+template <int HD, bool MASKED, typename L, bool GENERAL = false>
 static __device__ __forceinline__ void use_tile(const KVTile<HD>& T, int kb, int r, int g, int lo, int pos,
                                                 const uint4 (&qreg)[HD / 32], float scale2, float& m, L& l,
-                                                float4_t (&o)[HD / 16]) {
+                                                float4_t (&o)[HD / 16], float cap_in = 0.f, float cap_out = 0.f) {
   float4_t s[2];
   tile_scores<HD>(T.k, qreg, s);
-  tile_softmax_values<HD, MASKED, L>(s, T.v, T.vok, kb, r, g, lo, pos, scale2, m, l, o);
+  tile_softmax_values<HD, MASKED, L, GENERAL>(s, T.v, T.vok, kb, r, g, lo, pos, scale2, m, l, o, cap_in, cap_out);
 }
 
 // The same, choosing the variant: `pmin` and `lomax` are the smallest position and the largest
 // window start among the wave's rows (wave-uniform).
-template <int HD>
+template <int HD, bool GENERAL = false>
 static __device__ __forceinline__ void use_tile_auto(const KVTile<HD>& T, int kb, int r, int g, int lo, int pos,
                                                      int pmin, int lomax, const uint4 (&qreg)[HD / 32], float scale2,
-                                                     float& m, float& l, float4_t (&o)[HD / 16]) {
-  if (kb + 31 <= pmin && kb >= lomax) use_tile<HD, false, float>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o);
-  else use_tile<HD, true, float>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o);
+                                                     float& m, float& l, float4_t (&o)[HD / 16], float cap_in = 0.f,
+                                                     float cap_out = 0.f) {
+  if (kb + 31 <= pmin && kb >= lomax) use_tile<HD, false, float, GENERAL>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o, cap_in, cap_out);
+  else use_tile<HD, true, float, GENERAL>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o, cap_in, cap_out);
 }
 
 // out[t, h, :] from the chunks' partial results part_o [tokens, nh, num_splits, hd] and part_ml
 // [tokens, nh, num_splits, 2] (reference maximum in units of log2, sum), over the chunks that hold
-// keys visible from positions[t] (defined in attention_decode.hip).
+// keys visible from positions[t] (defined in attention_decode.hip). `sink`: the softmax has one more in its
+// denominator (a key of score 0 without a value), added once, here.
 int ts_launch_attention_combine(void* out, const float* part_o, const float* part_ml, const int32_t* positions,
                                 int num_tokens, int nh, int hd, int num_splits, int chunk, int window,
-                                hipStream_t stream);
+                                hipStream_t stream, int sink = 0);

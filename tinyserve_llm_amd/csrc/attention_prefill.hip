@@ -41,7 +41,8 @@ struct PrefillLds {
 // short prompt, which run alone at the end, then take a shorter step (2,048 tokens at head size 64:
 // 48.9 µs against 51.3; over long contexts the doubled reads of LDS cost more than that gains).
 // WHOLE: a page holds a multiple of 32 keys, so that every step lies in one page.
-template <int HD, int RT, int PRE_WAVES, bool WHOLE>
+// GENERAL: capped scores, weights in two terms (attention_mfma.h) and optionally a sink, added to a row's sum at the end.
+template <int HD, int RT, int PRE_WAVES, bool WHOLE, bool GENERAL>
 static __device__ __forceinline__ void
 prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -49,7 +50,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
              const int32_t* __restrict__ positions, const int32_t* __restrict__ tiles, int nh, int G, int page_size,
              int page_shift, int page_run, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
              float scale2, int window, float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits,
-             int chunk, int split) {
+             int chunk, int split, float cap_in, float cap_out, int sink) {
   constexpr int NC = HD / 32, NDB = HD / 16;   // operand registers of a 32-key step: 2 NC of K, NDB of V
   auto& stage = lds.stage;
   auto& wg_range = lds.range;
@@ -262,9 +263,9 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
         if constexpr (decltype(masked)::value) {
           // a step wholly beyond the tile's last position, or wholly before all its windows, has nothing for it
           if (kb <= tile_pmax[j] && kb + 31 >= tile_lomin[j])
-            use_tile<HD, true, float4_t>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j]);
+            use_tile<HD, true, float4_t, GENERAL>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j], cap_in, cap_out);
         } else {
-          use_tile<HD, false, float4_t>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j]);
+          use_tile<HD, false, float4_t, GENERAL>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j], cap_in, cap_out);
         }
       }
       __syncthreads();
@@ -290,11 +291,12 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = 4 * g + i;
-      const float lj = l[j][i];
+      float lj = l[j][i];
       const int rtk = (wave * RT + j) * tpt + row / G, rhh = row % G;
+      const float mj = __shfl(m[j], row, TS_WAVE);       // the row's reference maximum (lane `row` holds it)
+      if (GENERAL && sink && num_splits == 1 && lj > 0.f) lj += fast_exp2(-mj);   // the sink's score is 0
       if (num_splits > 1) {
         // the chunk's share of the row, not normalised: sums, and the reference maximum they are relative to
-        const float mj = __shfl(m[j], row, TS_WAVE);
         if (row / G < tpt && rtk < ntok) {
           const int64_t at = (((int64_t)(t0 + rtk) * nh + (int64_t)kvh * G + rhh) * num_splits + split);
 #pragma unroll
@@ -312,7 +314,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     }
 }
 
-template <int HD, int RT, int PRE_WAVES, bool WHOLE>
+template <int HD, int RT, int PRE_WAVES, bool WHOLE, bool GENERAL>
 __global__ void __launch_bounds__(PRE_WAVES * TS_WAVE)
 attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
@@ -320,7 +322,8 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
                          const int32_t* __restrict__ tiles, int num_tiles, int nh, int G, int dies_per_group,
                          int heads_per_group, int page_size, int page_shift, int page_run, int64_t kp, int64_t ks, int64_t kh,
                          int64_t vp, int64_t vh, int64_t vd, int max_blocks, float scale2, int window,
-                         float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits, int chunk) {
+                         float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits, int chunk,
+                         float cap_in, float cap_out, int sink) {
   __shared__ PrefillLds<HD> lds;
   // die = workgroup index mod 8. The dies form `groups` groups of `dies_per_group`, the heads as
   // many groups of `heads_per_group`; a group's (tile, head) pairs go round its dies, long tiles first.
@@ -329,9 +332,9 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
   if (item >= num_tiles * heads_per_group) return;
   const int tile = num_tiles - 1 - item / heads_per_group;
   const int kvh = (die / dies_per_group) * heads_per_group + item % heads_per_group;
-  prefill_tile<HD, RT, PRE_WAVES, WHOLE>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
+  prefill_tile<HD, RT, PRE_WAVES, WHOLE, GENERAL>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
                        G, page_size, page_shift, page_run, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml,
-                       num_splits, chunk, blockIdx.y);
+                       num_splits, chunk, blockIdx.y, cap_in, cap_out, sink);
 }
 
 // Keys: rows dense in head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages,
@@ -341,14 +344,19 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
 // takes every key from its start on) and the float workspaces part_o [num_tokens, nh, num_splits, hd] and
 // part_ml [num_tokens, nh, num_splits, 2]; every token from first_token on must then be in a tile (the ones
 // before it keep what `out` held). An entry of block_tables names 2^page_run consecutive pages of page_size keys.
-extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
-                                          const int32_t* block_tables, const int32_t* seq_of_token,
-                                          const int32_t* positions, const int32_t* tiles, int num_tiles,
-                                          int tile_tokens, int waves, int nh, int nkv, int hd, int page_size, int64_t kp,
-                                          int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
-                                          float scale, int window, int first_token, int num_tokens, int num_splits,
-                                          int chunk, float* part_o, float* part_ml, int page_run, hipStream_t stream) {
+static int launch_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
+                          const int32_t* block_tables, const int32_t* seq_of_token,
+                          const int32_t* positions, const int32_t* tiles, int num_tiles,
+                          int tile_tokens, int waves, int nh, int nkv, int hd, int page_size, int64_t kp,
+                          int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
+                          float scale, int window, int first_token, int num_tokens, int num_splits,
+                          int chunk, float* part_o, float* part_ml, int page_run, bool general, float softcap, int sink,
+                          hipStream_t stream) {
   if (num_tiles <= 0) return TS_OK;
+  if (general && (page_size % 32 || softcap < 0.f)) return TS_BAD_SHAPE;     // (the general variant walks whole steps only)
+  const float log2e = 1.44269504088896340736f;
+  const float cap_in = softcap > 0.f ? scale / softcap : 0.f, cap_out = softcap * log2e;
+  const float scale2 = softcap > 0.f ? 1.0f : scale * log2e;
   if (num_splits < 1 || num_splits > 65535) return TS_BAD_SHAPE;
   if (num_splits > 1 && (chunk <= 0 || chunk % 32 || !part_o || !part_ml || first_token < 0 || num_tokens <= first_token))
     return TS_BAD_SHAPE;
@@ -373,16 +381,17 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
   if (turns * 8 > 0x7fffffff) return TS_BAD_SHAPE;
   dim3 grid((unsigned)(8 * turns), num_splits);
 #define TS_PRE_W(HH, RR, WW)                                                                                    \
-  if (page_size % 32 == 0) TS_PRE_P(HH, RR, WW, true); else TS_PRE_P(HH, RR, WW, false)
-#define TS_PRE_P(HH, RR, WW, PP)                                                                                \
-  attn_prefill_mfma_kernel<HH, RR, WW, PP><<<grid, WW * TS_WAVE, 0, stream>>>(                                  \
+  if (general) { TS_PRE_P(HH, RR, WW, true, true); }                                                            \
+  else if (page_size % 32 == 0) { TS_PRE_P(HH, RR, WW, true, false); } else { TS_PRE_P(HH, RR, WW, false, false); }
+#define TS_PRE_P(HH, RR, WW, PP, GG)                                                                            \
+  attn_prefill_mfma_kernel<HH, RR, WW, PP, GG><<<grid, WW * TS_WAVE, 0, stream>>>(                              \
       (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,             \
       seq_of_token, positions, tiles, num_tiles, nh, G, dies_per_group, heads_per_group, page_size, page_shift, page_run, kp,  \
-      ks, kh, vp, vh, vd, max_blocks, scale * 1.44269504088896340736f, window, part_o, part_ml, num_splits, chunk)
+      ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml, num_splits, chunk, cap_in, cap_out, sink)
 #define TS_PRE_RT(HH)                                                                                           \
-  if (rt == 1) TS_PRE_W(HH, 1, 4); else if (rt == 2) TS_PRE_W(HH, 2, 4); else TS_PRE_W(HH, 4, 4)
+  if (rt == 1) { TS_PRE_W(HH, 1, 4) } else if (rt == 2) { TS_PRE_W(HH, 2, 4) } else { TS_PRE_W(HH, 4, 4) }
 #define TS_PRE_RT8(HH)                                                                                          \
-  if (rt == 1) TS_PRE_W(HH, 1, 8); else TS_PRE_W(HH, 2, 8)
+  if (rt == 1) { TS_PRE_W(HH, 1, 8) } else { TS_PRE_W(HH, 2, 8) }
   if (waves == 8) {
     switch (hd) {
       case 64: TS_PRE_RT8(64); break;
@@ -407,5 +416,33 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
   const int64_t skip = (int64_t)first_token * nh;     // rows of the tokens before the first listed one
   return ts_launch_attention_combine((bf16_t*)out + skip * hd, part_o + skip * num_splits * hd,
                                      part_ml + skip * num_splits * 2, positions + first_token,
-                                     num_tokens - first_token, nh, hd, num_splits, chunk, window, stream);
+                                     num_tokens - first_token, nh, hd, num_splits, chunk, window, stream, general ? sink : 0);
+}
+
+extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                          const int32_t* block_tables, const int32_t* seq_of_token,
+                                          const int32_t* positions, const int32_t* tiles, int num_tiles,
+                                          int tile_tokens, int waves, int nh, int nkv, int hd, int page_size, int64_t kp,
+                                          int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
+                                          float scale, int window, int first_token, int num_tokens, int num_splits,
+                                          int chunk, float* part_o, float* part_ml, int page_run, hipStream_t stream) {
+  return launch_prefill(out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, num_tiles, tile_tokens, waves, nh,
+                        nkv, hd, page_size, kp, ks, kh, vp, vh, vd, max_blocks, scale, window, first_token, num_tokens,
+                        num_splits, chunk, part_o, part_ml, page_run, false, 0.f, 0, stream);
+}
+
+// The same with capped scores (softcap > 0: cap * tanh(score / cap)), a sink (one more in the softmax's
+// denominator) and weights carried in two bfloat16 terms; pages of a multiple of 32 keys.
+extern "C" int ts_paged_attention_prefill_general(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                                  const int32_t* block_tables, const int32_t* seq_of_token,
+                                                  const int32_t* positions, const int32_t* tiles, int num_tiles,
+                                                  int tile_tokens, int waves, int nh, int nkv, int hd, int page_size,
+                                                  int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd,
+                                                  int max_blocks, float scale, int window, int first_token,
+                                                  int num_tokens, int num_splits, int chunk, float* part_o,
+                                                  float* part_ml, int page_run, float softcap, int sink,
+                                                  hipStream_t stream) {
+  return launch_prefill(out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, num_tiles, tile_tokens, waves, nh,
+                        nkv, hd, page_size, kp, ks, kh, vp, vh, vd, max_blocks, scale, window, first_token, num_tokens,
+                        num_splits, chunk, part_o, part_ml, page_run, true, softcap, sink, stream);
 }

@@ -52,6 +52,10 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_paged_attention_wave": [p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, i, i, i, p],
         "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, i, f,
                                       i, i, i, p],
+        "ts_paged_attention_decode_general": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, i, f,
+                                              i, i, f, i, p],
+        "ts_paged_attention_prefill_general": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i,
+                                               i, i, p, p, i, f, i, p],
         "ts_attention_combine": [p, p, p, p, i, i, i, i, i, i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
@@ -354,13 +358,16 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
                            seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, window: int = 0,
                            chunk: int | None = None, waves: int | None = None,
                            out: torch.Tensor | None = None, pages_per_entry: int = 1,
-                           leave_split: bool = False) -> "torch.Tensor | SplitAttention":
+                           leave_split: bool = False, softcap: float = 0.0, sink: bool = False
+                           ) -> "torch.Tensor | SplitAttention":
     """Split-key attention on the matrix cores for tokens that each bring one query (bfloat16,
     values in transposed pages). Every position in `positions` must lie inside the pages its row
     of `block_tables` has (checked by the caller on the host). `out`, if given, receives the result.
     `pages_per_entry`: as for `paged_attention_wave`. `leave_split`: where the keys are walked in
     2 to `SPLIT_ATTENTION_MAX_CHUNKS` chunks, the chunks' parts come back uncombined (a
-    `SplitAttention`), for the projection that reads them."""
+    `SplitAttention`), for the projection that reads them. `softcap` > 0 or `sink`: the kernel's
+    general variant (scores capped as softcap * tanh(score / softcap); one more in the softmax's
+    denominator; weights carried in two bfloat16 terms), which always combines."""
     _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
@@ -386,8 +393,16 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     if splits > 1:
         part_o = torch.empty((T, nh, splits, hd), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nh, splits, 2), dtype=torch.float32, device=q.device)
-    leave_split = leave_split and out is None and 1 < splits <= SPLIT_ATTENTION_MAX_CHUNKS
+    general = softcap > 0 or sink
+    leave_split = leave_split and not general and out is None and 1 < splits <= SPLIT_ATTENTION_MAX_CHUNKS
     out = None if leave_split else _out_like(q, out)
+    if general:
+        _run("paged_attention_decode_general", library().ts_paged_attention_decode_general(
+            _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+            _ptr(seq_of_token), _ptr(positions), T, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3],
+            v_cache.stride(0), v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], splits, chunk, waves,
+            float(scale), int(window), _page_run(pages_per_entry), float(softcap), int(sink), _stream()))
+        return out
     _run("paged_attention_decode", library().ts_paged_attention_decode(
         _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
         _ptr(seq_of_token), _ptr(positions), T, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3],
@@ -621,7 +636,7 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             seq_of_token: torch.Tensor, positions: torch.Tensor, tiles: torch.Tensor, scale: float,
                             window: int = 0, tile_tokens: int | None = None, out: torch.Tensor | None = None,
                             num_splits: int = 1, chunk: int = 0, first_token: int = 0, waves: int = PREFILL_WAVES,
-                            pages_per_entry: int = 1) -> torch.Tensor:
+                            pages_per_entry: int = 1, softcap: float = 0.0, sink: bool = False) -> torch.Tensor:
     """Attention of a packed step on the matrix cores (bfloat16, values in transposed pages).
     `tiles` int32 [num_tiles, 2] lists (first token, token count <= tile_tokens) per workgroup,
     every tile inside one request and inside the step (the caller built the list from the step's
@@ -631,7 +646,8 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     multiple of 32; the last takes every key from its start on) by workgroups of their own, and the
     chunks are combined afterwards: for steps of few tokens over long contexts, which have too few
     tiles to fill the chip. The tiles must then list every token from `first_token` on.
-    `pages_per_entry`: as for `paged_attention_wave`."""
+    `pages_per_entry`: as for `paged_attention_wave`. `softcap` > 0 or `sink`: the kernel's general
+    variant, as for `paged_attention_decode` (cache pages of a multiple of 32 keys)."""
     _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
@@ -659,31 +675,41 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         _need(num_splits <= MAX_DECODE_SPLITS, lambda: f"at most {MAX_DECODE_SPLITS} chunks")
         part_o = torch.empty((T, nh, num_splits, hd), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nh, num_splits, 2), dtype=torch.float32, device=q.device)
-    _run("paged_attention_prefill", library().ts_paged_attention_prefill(
-        _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
-        _ptr(tiles), tiles.shape[0], tile_tokens, waves, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
-        v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], float(scale), int(window), first_token, T,
-        num_splits, chunk, _ptr(part_o), _ptr(part_ml), _page_run(pages_per_entry), _stream()))
+    args = (_ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
+            _ptr(tiles), tiles.shape[0], tile_tokens, waves, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
+            v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], float(scale), int(window), first_token, T,
+            num_splits, chunk, _ptr(part_o), _ptr(part_ml), _page_run(pages_per_entry))
+    if softcap > 0 or sink:
+        _need(k_cache.shape[1] % 32 == 0, "the general variant takes cache pages of a multiple of 32 keys")
+        _run("paged_attention_prefill_general", library().ts_paged_attention_prefill_general(*args, float(softcap), int(sink), _stream()))
+    else:
+        _run("paged_attention_prefill", library().ts_paged_attention_prefill(*args, _stream()))
     return out
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int,
-                    scale: float, window: int = 0, leave_split: bool = False) -> "torch.Tensor | SplitAttention":
+                    scale: float, window: int = 0, leave_split: bool = False, softcap: float = 0.0,
+                    sink: bool = False) -> "torch.Tensor | SplitAttention":
     """Attention of a packed step over the cache; picks the kernel for the storage type and shape.
     float32 always takes the one-wave-per-row kernel, whose sums do not depend on the batch;
     bfloat16 takes the matrix-core kernels where they serve the shape. `leave_split`: a step of single
-    tokens whose keys are walked in chunks may come back as a `SplitAttention` (see `paged_attention_decode`)."""
+    tokens whose keys are walked in chunks may come back as a `SplitAttention` (see `paged_attention_decode`).
+    `softcap` > 0 (scores capped as softcap * tanh(score / softcap)) or `sink` (one more in the softmax's
+    denominator) choose the kernels' general variants; those, and value rows of a size of their own, fall
+    back to `paged_attention_general`, which is 32-bit throughout."""
+    general = softcap > 0 or sink
     tables = ctx.block_tables[space]
     # (the tables count in pages of ctx.page_size tokens; the pools may be cut into shorter ones)
     table_page = getattr(ctx, "page_size", 0) or k_cache.shape[1]
     _need(table_page % k_cache.shape[1] == 0, lambda: f"block tables in pages of {table_page} over a cache in pages of {k_cache.shape[1]}")
     per_entry = table_page // k_cache.shape[1]
-    if decode_kernel_takes(q, k_cache, v_cache):
+    if (k_cache.shape[3] == v_cache.shape[3] and decode_kernel_takes(q, k_cache, v_cache)
+            and (not general or k_cache.shape[1] % 32 == 0)):
         capacity = tables.shape[1] * table_page
         decode_ok = -(-capacity // 1024) <= MAX_DECODE_SPLITS and q.shape[0] <= MAX_DECODE_TOKENS
         if ctx.max_query_len == 1 and decode_ok:
             return paged_attention_decode(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window,
-                                          pages_per_entry=per_entry, leave_split=leave_split)
+                                          pages_per_entry=per_entry, leave_split=leave_split, softcap=softcap, sink=sink)
         # the one-token requests that lead the step go to the split-key kernel, the rest to the tiles
         cu = ctx.host_cu_seqlens
         lead = 0
@@ -702,11 +728,14 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         out = torch.empty_like(q)
         if lead:
             paged_attention_decode(q[:lead], k_cache, v_cache, tables, ctx.seq_of_token[:lead], ctx.positions[:lead],
-                                   scale, window, out=out[:lead], pages_per_entry=per_entry)
+                                   scale, window, out=out[:lead], pages_per_entry=per_entry, softcap=softcap, sink=sink)
         splits, chunk = prefill_splits(tiles.shape[0] * nkv, max(ctx.host_context_lens[lead:], default=0))
         return paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale,
                                        window, tile_tokens=tile_tokens, out=out, num_splits=splits, chunk=chunk,
-                                       first_token=cu[lead], waves=waves, pages_per_entry=per_entry)
+                                       first_token=cu[lead], waves=waves, pages_per_entry=per_entry, softcap=softcap, sink=sink)
+    if general or k_cache.shape[3] != v_cache.shape[3]:
+        return paged_attention_general(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, softcap=softcap,
+                                       sink=sink, window=window, pages_per_entry=per_entry)
     return paged_attention_wave(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window,
                                 pages_per_entry=per_entry)
 
@@ -1674,15 +1703,3 @@ def paged_attention_general(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         T, nh, nkv, hd, vd, k_cache.shape[1], *k_cache.stride()[:3], *v_cache.stride(), block_tables.shape[1],
         float(scale), float(softcap), int(sink), int(window), _code(q.dtype), _page_run(pages_per_entry), _stream()))
     return out
-
-
-def attention_general(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int, scale: float, *,
-                      softcap: float = 0.0, sink: bool = False, window: int = 0) -> torch.Tensor:
-    """Attention of a packed step over the cache for mixers with capped scores, a sink or values of
-    their own size; picks the kernel for the storage type and shape."""
-    tables = ctx.block_tables[space]
-    table_page = getattr(ctx, "page_size", 0) or k_cache.shape[1]
-    _need(table_page % k_cache.shape[1] == 0, lambda: f"block tables in pages of {table_page} over a cache in pages of {k_cache.shape[1]}")
-    per_entry = table_page // k_cache.shape[1]
-    return paged_attention_general(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, softcap=softcap,
-                                   sink=sink, window=window, pages_per_entry=per_entry)

@@ -131,7 +131,9 @@ class GeneralAttention(Mixer):
     softcap * tanh(score / softcap), and a softmax with a sink (one more in the denominator).
     Separate q, k, v weights of a checkpoint land in row slices of one fused projection, whose output,
     like the output projection's, is 32-bit; rotation, norms, scores and weights are 32-bit in every
-    storage type (`hip.qkv_finish`, `hip.paged_attention_general`)."""
+    storage type (`hip.qkv_finish`, `hip.paged_attention_general`); in bfloat16, where key and value heads
+    have one of the matrix-core kernels' sizes, those kernels' general variants run instead, which cap
+    in 32-bit and carry the weights into the products in two bfloat16 terms."""
 
     graph_safe = True
 
@@ -187,7 +189,7 @@ class GeneralAttention(Mixer):
                            self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, x.dtype,
                            interleaved=getattr(enc, "interleaved", True), qk_norm_eps=self.qk_norm_eps,
                            v_norm_eps=self.v_norm_eps)
-        o = hip.attention_general(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, softcap=self.softcap,
-                                  sink=self.sink, window=self.window)
+        o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window, softcap=self.softcap,
+                                sink=self.sink)
         return linear(o.view(ctx.num_tokens, self.num_heads * self.value_dim), self.o, out_dtype=torch.float32,
                       packed=self.o_packed)
