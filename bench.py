@@ -12,6 +12,16 @@ times the kernels of one decode step class by class (qkv, attention, o, gate|up,
 sampling) with events around each launch of an eager step, and prints the bytes each class has to
 read, its time and its rate beside the step's total, as one JSON line.
 
+    python bench.py --designs [--shape 1b|3b] [--layers L]
+
+measures the Rugezen decoder (parallel layers on a 32-bit stream, attention with head norms, capped
+scores and a sink, a minGRU every fourth layer, dense squared-relu feed-forward) beside the Llama
+decoder at equal layer sizes and equal parameter count, random weights: prefill tokens/s and decode
+tokens/s at batch 1, 8 and 64 through the whole engine, and kernel by kernel the pairs of like kernels
+(attention over prompt portions and over decoded tokens, rotation and cache write, residual sum and
+norms, the feed-forward's activation) with the bytes or operations each has to move and what share of
+the machine's peak that comes to. One JSON line.
+
     python bench.py --scenario requests-3b | chunked-8b [--layers L]
 
 runs a whole workload through `LLM.generate` instead and prints one JSON line of its own: many
@@ -140,6 +150,196 @@ def scenario(name: str, layers: int | None, dtype_name: str) -> int:
     return 0
 
 
+def designs(args) -> int:
+    """The Rugezen decoder beside the Llama decoder at the layer sizes of `--shape`: whole-engine
+    throughput, and the like kernels of the two side by side. One JSON line."""
+    import torch
+
+    from tinyserve_llm_amd.config import LlamaConfig, RopeScaling
+    from tinyserve_llm_amd.config.rugezen import RugezenAttention, RugezenConfig, RugezenLayer, RugezenMinGRU
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.loading import random_model
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    from tinyserve_llm_amd.ops import hip
+    from tinyserve_llm_amd.parts.base import StepContext
+
+    sizes = SHAPES[args.shape]
+    sh = sizes["shape"]
+    layers = args.layers or sizes["layers_full"]
+    hidden, nh, nkv, hd, inter, vocab = (sh["hidden_size"], sh["num_attention_heads"], sh["num_key_value_heads"], sh["head_dim"],
+                                         sh["intermediate_size"], sh["vocab_size"])
+    llama = LlamaConfig(num_hidden_layers=layers, rope_scaling=RopeScaling(**{**ROPE, "factor": sizes["rope_factor"]}), **sh)
+    att = RugezenAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, rot_dims=hd // 2, rot_base=sh["rope_theta"], scale=hd ** -0.5,
+                           softcap=50.0)
+    ff = 3 * inter // 2                  # two matrices of this width hold what the gated feed-forward's three hold
+    rug = RugezenConfig(vocab=vocab, width=hidden, norm_eps=1e-5, residual_mult=0.5, layers=tuple(
+        RugezenLayer("mingru", RugezenMinGRU(width=hidden), ff) if i % 4 == 2 else RugezenLayer("attention", att, ff)
+        for i in range(layers)))
+    prompt_len = args.context
+    max_model_len = max(MAX_MODEL_LEN, prompt_len + 1024)
+    rng = random.Random(0)
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def whole_engine(config) -> dict:
+        model = random_model(config, 0, torch.bfloat16, "cuda:0")
+        out = {"parameters": sum(t.numel() for t in (getattr(part, name) for layer in model.layers
+                                                     for part in layer.parts().values() for name in part.param_specs()))}
+
+        def engine(batch):
+            pages = batch * -(-max_model_len // PAGE) + 2
+            sc = SchedulerConfig(max_model_len=max_model_len, max_num_seqs=batch,
+                                 max_num_batched_tokens=max(prompt_len, batch + 1) + batch, watermark=0.0)
+            return LLM(None, sc, CacheConfig(block_size=PAGE, caching=False), dtype=torch.bfloat16, num_blocks=pages, seed=0,
+                       model=model)
+        llm = engine(1)
+        times = []
+        for r in range(3):
+            llm.add_request([rng.randrange(vocab) for _ in range(prompt_len)], SamplingParams(max_tokens=1, temperature=0.0, ignore_eos=True))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            llm.step()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        out["prefill_tok_s"] = prompt_len / min(times[1:])
+        del llm
+        for batch in (1, 8, 64):
+            llm = engine(batch)
+            sp = SamplingParams(max_tokens=max_model_len - prompt_len, temperature=0.0, ignore_eos=True)
+            for _ in range(batch):
+                llm.add_request([rng.randrange(vocab) for _ in range(prompt_len)], sp)
+            while any(q.in_prefill or not q.output_token_ids for q in llm.scheduler.running + llm.scheduler.waiting):
+                llm.step()
+            for _ in range(6):
+                llm.step()
+            steps = 32
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                llm.step()
+            torch.cuda.synchronize()
+            out[f"decode_b{batch}_tok_s"] = batch * steps / (time.perf_counter() - t0)
+            del llm
+        del model
+        torch.cuda.empty_cache()
+        return out
+
+    def replayed(fn, reps: int) -> float:
+        fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            kept = fn()
+        best = float("inf")
+        for _ in range(reps):
+            sweep.sum()
+            begin.record()
+            graph.replay()
+            end.record()
+            end.synchronize()
+            best = min(best, 1e3 * begin.elapsed_time(end))
+        del kept, graph
+        return best
+
+    overhead = []
+
+    def timed(fn, reps: int = 5) -> float:
+        """Microseconds of the best of `reps` replays of `fn` recorded into a graph (what the host does
+        between launches is then not in the time), each after a sweep of the caches, less what the replay of
+        a graph of one tiny kernel takes."""
+        if not overhead:
+            tiny = torch.zeros(64, dtype=torch.int32, device="cuda")
+            overhead.append(replayed(lambda: tiny.add_(1), reps))
+        return max(replayed(fn, reps) - overhead[0], 1e-3)
+
+    sweep = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    bf = torch.bfloat16
+
+    def context(starts, counts, pool_page):
+        positions, seq_of, cu, tables = [], [], [0], []
+        per = -(-max(a + b for a, b in zip(starts, counts)) // PAGE)
+        for i, (s0, n) in enumerate(zip(starts, counts)):
+            positions += list(range(s0, s0 + n))
+            seq_of += [i] * n
+            cu.append(cu[-1] + n)
+            tables.append(list(range(i * per, (i + 1) * per)))
+        ends = [a + b for a, b in zip(starts, counts)]
+        ctx = StepContext(num_tokens=len(positions), num_seqs=len(starts), token_ids=dev([0] * len(positions)), positions=dev(positions),
+                          seq_of_token=dev(seq_of), cu_seqlens=dev(cu), context_lens=dev(ends), state_slots=dev(list(range(len(starts)))),
+                          slot_mapping=[], block_tables=[dev(tables)], host_cu_seqlens=cu, host_starts=list(starts),
+                          host_context_lens=ends, host_state_slots=list(range(len(starts))), page_size=PAGE)
+        slots = dev([tables[i][p // PAGE] * PAGE + p % PAGE for i, p in zip(seq_of, positions)])
+        return ctx, slots, len(starts) * per * (PAGE // pool_page)
+
+    def kernel_pairs() -> dict:
+        pairs = {}
+        pool_page = 32
+        mfma = hip.measure_peaks()
+        read_peak, mfma_peak = mfma["read_GBps"] * 1e9, mfma["mfma_bf16_TFLOPs"] * 1e12
+        for label, starts, counts in (("prompt portion", [0], [prompt_len]), ("decoded tokens, batch 64", [prompt_len] * 64, [1] * 64)):
+            ctx, slots, pages = context(starts, counts, pool_page)
+            T = ctx.num_tokens
+            k = torch.randn(pages, nkv, pool_page, hd, device="cuda").to(bf).permute(0, 2, 1, 3)
+            v = torch.randn(pages, nkv, hd, pool_page, device="cuda").to(bf).permute(0, 3, 1, 2)
+            q = torch.randn(T, nh, hd, device="cuda").to(bf)
+            keys = sum(n * (s0 + (n + 1) / 2) for s0, n in zip(starts, counts))
+            flops = 4 * nh * hd * keys
+            nbytes = sum(s0 + n for s0, n in zip(starts, counts)) * 2 * nkv * hd * 2
+            plain_us = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5))
+            general_us = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5, softcap=50.0, sink=True))
+            if T > 64:
+                pairs[f"attention, {label}"] = {"llama_us": plain_us, "rugezen_us": general_us, "flops": flops,
+                                                "llama_frac_of_mfma": flops / plain_us * 1e6 / mfma_peak,
+                                                "rugezen_frac_of_mfma": flops / general_us * 1e6 / mfma_peak}
+            else:
+                pairs[f"attention, {label}"] = {"llama_us": plain_us, "rugezen_us": general_us, "bytes": nbytes,
+                                                "llama_frac_of_read": nbytes / plain_us * 1e6 / read_peak,
+                                                "rugezen_frac_of_read": nbytes / general_us * 1e6 / read_peak}
+            # rotation and cache write: bfloat16 q|k|v rows in, against 32-bit rows in with the head norms
+            row = (nh + 2 * nkv) * hd
+            table = torch.randn(max_model_len, hd, device="cuda")
+            freqs = torch.rand(hd // 4, dtype=torch.float64, device="cuda")
+            qkv16, qkv32 = torch.randn(T, row, device="cuda").to(bf), torch.randn(T, row, device="cuda")
+            us_a = timed(lambda: hip.rope_store(qkv16, table, ctx.positions, slots, k, v, nh, nkv, hd))
+            us_b = timed(lambda: hip.qkv_finish(qkv32, freqs, ctx.positions, slots, k, v, nh, nkv, hd, hd, bf, qk_norm_eps=1e-5, v_norm_eps=1e-5))
+            bytes_a, bytes_b = T * row * 2 * 2, T * row * (4 + 2)
+            pairs[f"rotation and cache write, {label}"] = {"llama_us": us_a, "rugezen_us": us_b, "llama_bytes": bytes_a, "rugezen_bytes": bytes_b,
+                                                           "llama_frac_of_read": bytes_a / us_a * 1e6 / read_peak,
+                                                           "rugezen_frac_of_read": bytes_b / us_b * 1e6 / read_peak}
+            # residual sum and norm: bfloat16 stream and one norm, against the 32-bit stream, two branches and two norms
+            x16, r16 = (torch.randn(T, hidden, device="cuda").to(bf) for _ in range(2))
+            w16 = torch.ones(hidden, device="cuda").to(bf)
+            x32, a32, b32 = (torch.randn(T, hidden, device="cuda") for _ in range(3))
+            us_a = timed(lambda: hip.rmsnorm(x16, w16, 1e-5, r16))
+            us_b = timed(lambda: hip.stream_update_norm(x32, a32, b32, w16, 0.5, (w16, w16), 1e-5, out_dtype=bf))
+            bytes_a, bytes_b = T * hidden * 2 * 4, T * hidden * (4 * 4 + 2 * 2)
+            pairs[f"residual sum and norms, {label}"] = {"llama_us": us_a, "rugezen_us": us_b, "llama_bytes": bytes_a, "rugezen_bytes": bytes_b,
+                                                         "llama_frac_of_read": bytes_a / us_a * 1e6 / read_peak,
+                                                         "rugezen_frac_of_read": bytes_b / us_b * 1e6 / read_peak}
+            gu, up, bias = torch.randn(T, 2 * inter, device="cuda").to(bf), torch.randn(T, ff, device="cuda"), torch.randn(ff, device="cuda").to(bf)
+            us_a = timed(lambda: hip.silu_mul(gu))
+            us_b = timed(lambda: hip.bias_activation(up, bias, "relu2", bf))
+            bytes_a, bytes_b = T * inter * 2 * 3, T * ff * (4 + 2)
+            pairs[f"feed-forward activation, {label}"] = {"llama_us": us_a, "rugezen_us": us_b, "llama_bytes": bytes_a, "rugezen_bytes": bytes_b,
+                                                          "llama_frac_of_read": bytes_a / us_a * 1e6 / read_peak,
+                                                          "rugezen_frac_of_read": bytes_b / us_b * 1e6 / read_peak}
+            zxg, state = torch.randn(T, 3 * hidden, device="cuda"), torch.zeros(len(starts), hidden, device="cuda")
+            us_b = timed(lambda: hip.mingru_scan(zxg, bias[:2 * hidden].contiguous() if ff >= 2 * hidden else None, state, ctx.cu_seqlens,
+                                                 ctx.state_slots, max(counts), bf))
+            bytes_b = T * hidden * (3 * 4 + 2)
+            pairs[f"minGRU scan, {label}"] = {"rugezen_us": us_b, "rugezen_bytes": bytes_b, "rugezen_frac_of_read": bytes_b / us_b * 1e6 / read_peak}
+        pairs["peaks"] = {"read_GBps": read_peak / 1e9, "mfma_bf16_TFLOPs": mfma_peak / 1e12}
+        return pairs
+
+    record = {"designs": {"llama": whole_engine(llama), "rugezen": whole_engine(rug)}, "kernels": kernel_pairs(),
+              "config": {"shape": args.shape, "layers": layers, "hidden": hidden, "heads": nh, "kv_heads": nkv, "head_dim": hd,
+                         "llama_intermediate": inter, "rugezen_ff": ff, "rugezen_mingru_every": 4, "vocab": vocab,
+                         "context": prompt_len, "dtype": "bf16", "data": "synthetic uniform token ids, random weights"}}
+    print(json.dumps(record))
+    return 0
+
+
 def kernel_classes(llm, config, batch: int, reps: int = 5) -> dict:
     """Times one decode step's kernels by class. An eager step (no graph) is run once with every
     launch of the engine's kernel module noted down with its operands; then each class's launches
@@ -264,6 +464,9 @@ def main() -> int:
                     help="'prefill': time the 2,048-token prefill alone and print its record (for profiling)")
     ap.add_argument("--scenario", default=None, choices=sorted(SCENARIOS),
                     help="run a whole workload through LLM.generate instead of the decode step")
+    ap.add_argument("--designs", action="store_true",
+                    help="measure the Rugezen decoder beside the Llama decoder at the layer sizes of --shape: whole-engine "
+                         "throughput and the like kernels side by side; one JSON line")
     ap.add_argument("--kernel-classes", action="store_true",
                     help="time one decode step's kernels class by class (bytes, microseconds, GB/s) and exit")
     ap.add_argument("--peaks", action="store_true",
@@ -287,6 +490,8 @@ def main() -> int:
         return 0
     if args.scenario:
         return scenario(args.scenario, args.layers, args.dtype)
+    if args.designs:
+        return designs(args)
     sizes = SHAPES[args.shape]
     full_layers = sizes["layers_full"]
     args.layers = args.layers or full_layers

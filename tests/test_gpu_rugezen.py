@@ -116,19 +116,24 @@ def test_mingru_scan_over_unequal_requests_and_steps(in_dtype, width):
         lengths = [2, 1, 1, 64, 33]
 
 
-def test_mingru_stretches_equal_the_plain_walk_closely():
-    """The same portion walked by one wave and cut into sixteen stretches: 32-bit rounding apart."""
+@pytest.mark.parametrize("n", [100, 127, 128, 129, 1024])
+def test_mingru_cuts_equal_the_plain_walk_closely(n):
+    """The same portion walked by one wave, cut into stretches for the waves of one workgroup (fewer than
+    128 tokens), and cut into chunks of 32 for two kernels (from 128 on): 32-bit rounding apart."""
     h = hip()
-    width, n = 64, 1024
+    width = 200
     zxg = (torch.randn(n, 3 * width) * 2).to(DEV)
     cu = torch.tensor([0, n], dtype=torch.int32, device=DEV)
-    slot = torch.tensor([0], dtype=torch.int32, device=DEV)
-    s1, s2 = torch.zeros(1, width, device=DEV), torch.zeros(1, width, device=DEV)
-    one = h.mingru_scan(zxg, None, s1, cu, slot, 1, torch.float32)        # (told 1: a single wave)
+    slot = torch.tensor([1], dtype=torch.int32, device=DEV)
+    s1 = torch.rand(2, width, device=DEV)
+    s2 = s1.clone()
+    # (told 1: a single wave; the kernel walks the whole portion whatever it is told)
+    one = h.mingru_scan(zxg, None, s1, cu, slot, 1, torch.float32)
     cut = h.mingru_scan(zxg, None, s2, cu, slot, n, torch.float32)
-    assert h.mingru_waves(1) == 1 and h.mingru_waves(n) == 16
+    assert h.mingru_waves(1) == 1 and h.mingru_waves(127) == 3 and h.MINGRU_CHUNKS_FROM == 128
     torch.testing.assert_close(cut, one, atol=2e-6, rtol=1e-5)
     torch.testing.assert_close(s2, s1, atol=2e-6, rtol=1e-5)
+    assert torch.equal(s2[0], s1[0])
 
 
 # ---- rotation, head norms and the cache write; attention over pages ----------------------------

@@ -85,6 +85,66 @@ stream_update_norm_kernel(float* __restrict__ x, const void* __restrict__ a, int
   }
 }
 
+// The same for rows of up to RS_THREADS * HELD elements whose branches are 32-bit and whose norms' weights, bias and
+// outputs share the type H: every load of the row goes out before the first is used (no branch on a storage type
+// or on whether an operand is there stands between two loads: an operand that is not there is read from another of
+// its shape and counts times 0), and the updated row stays in registers between the sum of squares and the scaling.
+#define RS_HELD 16
+template <typename H, int HELD, bool NORMS>
+__global__ void __launch_bounds__(RS_THREADS)
+stream_update_norm_held_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b,
+                               const H* __restrict__ bias, float mult, H* __restrict__ h1, H* __restrict__ h2,
+                               const H* __restrict__ w1, const H* __restrict__ w2, float eps,
+                               const int32_t* __restrict__ rows, int width) {
+  __shared__ float scratch[RS_THREADS / TS_WAVE];
+  const int64_t r = blockIdx.x;
+  const int64_t t = rows ? rows[r] : r;
+  float* xr = x + t * width;
+  const bool update = a || b, bias_on = bias && update;
+  // an operand that is not there is read from another of its size (the row itself; a norm's weight) and not used
+  const float* ar = (a ? a : x) + t * width;
+  const float* br = (b ? b : x) + t * width;
+  const H* wa = w1 ? w1 : w2;
+  const H* wb = w2 ? w2 : w1;
+  const H* bs = bias ? bias : (NORMS ? wa : (const H*)xr);
+  float v[HELD], va[HELD], vb[HELD], vbias[HELD], wva[HELD], wvb[HELD];
+#pragma unroll
+  for (int j = 0; j < HELD; ++j) {
+    const int i = min(threadIdx.x + j * RS_THREADS, width - 1);     // (a lane beyond the row reads its last element, and stores nothing)
+    v[j] = xr[i];
+    va[j] = ar[i];
+    vb[j] = br[i];
+    vbias[j] = Num<H>::ld(bs + i);
+    if constexpr (NORMS) {
+      wva[j] = Num<H>::ld(wa + i);
+      wvb[j] = Num<H>::ld(wb + i);
+    }
+  }
+  float squares = 0.f;
+#pragma unroll
+  for (int j = 0; j < HELD; ++j) {
+    const int i = threadIdx.x + j * RS_THREADS;
+    // x + mult * (a + b + bias), the sum of the branches first
+    const float add = (a ? va[j] : 0.f) + (b ? vb[j] : 0.f) + (bias_on ? vbias[j] : 0.f);
+    v[j] = update ? fmaf(mult, add, v[j]) : v[j];
+    if (update && i < width) xr[i] = v[j];
+    squares = i < width ? fmaf(v[j], v[j], squares) : squares;
+  }
+  if constexpr (NORMS) {
+    const float total = block_sum(squares, scratch);
+    const float inv = 1.0f / sqrtf(total / (float)width + eps);
+#pragma unroll
+    for (int j = 0; j < HELD; ++j) {
+      const int i = threadIdx.x + j * RS_THREADS;
+      if (i < width) {
+        const float n = v[j] * inv;
+        if (h1) Num<H>::st(h1 + r * width + i, n * wva[j]);
+        if (h2) Num<H>::st(h2 + r * width + i, n * wvb[j]);
+      }
+    }
+  }
+}
+
 extern "C" int ts_stream_update_norm(float* x, const void* a, int a_dtype, const void* b, int b_dtype, const void* bias,
                                      int bias_dtype, float mult, void* h1, void* h2, int h_dtype, const void* w1,
                                      const void* w2, int w_dtype, float eps, const int32_t* rows, int num_rows, int width,
@@ -93,6 +153,22 @@ extern "C" int ts_stream_update_norm(float* x, const void* a, int a_dtype, const
   if (width <= 0 || !x || (rows && (a || b)) || (h1 && !w1) || (h2 && !w2)) return TS_BAD_SHAPE;
   for (int code : {a_dtype, b_dtype, bias_dtype, h_dtype, w_dtype})
     if (code != 0 && code != 1) return TS_BAD_DTYPE;
+  const bool typed = (!a || a_dtype == 0) && (!b || b_dtype == 0) && width <= RS_THREADS * RS_HELD &&
+                     (!bias || bias_dtype == h_dtype || !(h1 || h2)) && (!(h1 || h2) || w_dtype == h_dtype);
+  if (typed) {
+    const int code = (h1 || h2) ? h_dtype : bias_dtype;
+#define RS_TYPED_N(H, HELD, NN) \
+  stream_update_norm_held_kernel<H, HELD, NN><<<num_rows, RS_THREADS, 0, stream>>>(x, (const float*)a, (const float*)b, \
+      (const H*)bias, mult, (H*)h1, (H*)h2, (const H*)w1, (const H*)w2, eps, rows, width)
+#define RS_TYPED(H, HELD) if (h1 || h2) { RS_TYPED_N(H, HELD, true); } else { RS_TYPED_N(H, HELD, false); }
+#define RS_TYPED_H(H) \
+  if (width <= RS_THREADS * 4) { RS_TYPED(H, 4); } else if (width <= RS_THREADS * 8) { RS_TYPED(H, 8); } else { RS_TYPED(H, RS_HELD); }
+    if (code == 0) { RS_TYPED_H(float) } else { RS_TYPED_H(bf16_t) }
+#undef RS_TYPED_H
+#undef RS_TYPED
+#undef RS_TYPED_N
+    return ts_check_launch();
+  }
   stream_update_norm_kernel<<<num_rows, RS_THREADS, 0, stream>>>(x, a, a_dtype, b, b_dtype, bias, bias_dtype, mult, h1, h2,
                                                                  h_dtype, w1, w2, w_dtype, eps, rows, width);
   return ts_check_launch();
@@ -119,6 +195,31 @@ bias_activation_kernel(void* __restrict__ out, int out_code, const void* __restr
   }
 }
 
+// Four elements a thread (rows of a multiple of four elements, 16-byte aligned 32-bit input, bfloat16 or 32-bit output).
+template <typename TO>
+__global__ void __launch_bounds__(RS_THREADS)
+bias_activation_by4_kernel(TO* __restrict__ out, const float* __restrict__ in, const void* __restrict__ bias, int bias_code,
+                           int64_t fours, int width, int act) {
+  for (int64_t idx = (int64_t)blockIdx.x * RS_THREADS + threadIdx.x; idx < fours; idx += (int64_t)gridDim.x * RS_THREADS) {
+    const int i = (int)((idx * 4) % width);
+    const float4 z4 = *(const float4*)(in + idx * 4);
+    float z[4] = {z4.x, z4.y, z4.z, z4.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (bias) z[k] += rs_load(bias, bias_code, i + k);
+      z[k] = rs_activate(z[k], act);
+    }
+    if constexpr (sizeof(TO) == 4) {
+      *(float4*)((float*)out + idx * 4) = make_float4(z[0], z[1], z[2], z[3]);
+    } else {
+      uint2 packed;
+      packed.x = (uint32_t)f2bf(z[0]) | ((uint32_t)f2bf(z[1]) << 16);
+      packed.y = (uint32_t)f2bf(z[2]) | ((uint32_t)f2bf(z[3]) << 16);
+      *(uint2*)((bf16_t*)out + idx * 4) = packed;
+    }
+  }
+}
+
 extern "C" int ts_bias_activation(void* out, int out_dtype, const void* in, int in_dtype, const void* bias, int bias_dtype,
                                   int num_rows, int width, int act, hipStream_t stream) {
   if (num_rows <= 0) return TS_OK;
@@ -126,6 +227,18 @@ extern "C" int ts_bias_activation(void* out, int out_dtype, const void* in, int 
   for (int code : {out_dtype, in_dtype, bias_dtype})
     if (code != 0 && code != 1) return TS_BAD_DTYPE;
   const int64_t total = (int64_t)num_rows * width;
+  if (in_dtype == 0 && width % 4 == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0) {
+    const int64_t fours = total / 4;
+    int64_t groups = (fours + RS_THREADS - 1) / RS_THREADS;
+    if (groups > 16384) groups = 16384;
+    if (out_dtype == 0)
+      bias_activation_by4_kernel<float><<<(unsigned)groups, RS_THREADS, 0, stream>>>((float*)out, (const float*)in, bias, bias_dtype,
+                                                                                    fours, width, act);
+    else
+      bias_activation_by4_kernel<bf16_t><<<(unsigned)groups, RS_THREADS, 0, stream>>>((bf16_t*)out, (const float*)in, bias, bias_dtype,
+                                                                                     fours, width, act);
+    return ts_check_launch();
+  }
   int64_t blocks = (total + RS_THREADS - 1) / RS_THREADS;
   if (blocks > 16384) blocks = 16384;
   bias_activation_kernel<<<(unsigned)blocks, RS_THREADS, 0, stream>>>(out, out_dtype, in, in_dtype, bias, bias_dtype, total,

@@ -81,6 +81,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_stream_update_norm": [p, p, i, p, i, p, i, f, p, p, i, p, p, i, f, p, i, i, p],
         "ts_bias_activation": [p, i, p, i, p, i, i, i, i, p],
         "ts_mingru_scan": [p, i, p, i, p, i, p, p, p, i, i, i, p],
+        "ts_mingru_scan_chunks": [p, i, p, i, p, i, p, p, p, p, p, i, i, i, p],
         "ts_qkv_finish": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, f, i, f, i, i64, i64, i64, i64, i64, i64, i64, i, i, p],
         "ts_paged_attention_general": [p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, f, i, i,
                                        i, i, p],
@@ -1597,6 +1598,8 @@ def bias_activation(x: torch.Tensor, bias: torch.Tensor | None, activation: str,
 
 MINGRU_STRETCH = 32       # tokens of a request's portion per wave from which the scan is cut into stretches
 MINGRU_MAX_WAVES = 16
+MINGRU_CHUNKS_FROM = 128  # tokens of the longest portion from which the scan runs as two kernels over chunks of 32
+MINGRU_CHUNK = 32
 
 
 def mingru_waves(longest: int) -> int:
@@ -1609,7 +1612,8 @@ def mingru_scan(zxg: torch.Tensor, bias: torch.Tensor | None, state: torch.Tenso
     """The minGRU recurrence over a packed step: zxg [tokens, 3 width] holds the projected z | x | g
     rows, bias [2 width] the biases of z and x; request s owns tokens cu_seqlens[s] .. cu_seqlens[s+1]
     and the float32 state row state[state_slots[s]], which the step advances. Returns
-    S_t * silu(g_t) [tokens, width] in `out_dtype`. `longest`: the most tokens any request feeds."""
+    S_t * silu(g_t) [tokens, width] in `out_dtype`. `longest`: the most tokens any request feeds (no
+    request may feed more: the kernels' cut of the work follows it)."""
     _gpu(zxg, bias, state, cu_seqlens, state_slots)
     _need(zxg.dim() == 2 and zxg.shape[1] % 3 == 0 and zxg.is_contiguous(), "zxg must be contiguous [tokens, 3 width]")
     width = zxg.shape[1] // 3
@@ -1621,6 +1625,14 @@ def mingru_scan(zxg: torch.Tensor, bias: torch.Tensor | None, state: torch.Tenso
     _need(cu_seqlens.dtype == torch.int32 and cu_seqlens.shape == (num_seqs + 1,) and cu_seqlens.is_contiguous(),
           "cu_seqlens must be int32 [requests + 1]")
     out = torch.empty((zxg.shape[0], width), dtype=out_dtype, device=zxg.device)
+    if longest >= MINGRU_CHUNKS_FROM:
+        chunks = -(-longest // MINGRU_CHUNK)
+        folds = torch.empty((num_seqs, chunks, width, 2), dtype=torch.float32, device=zxg.device)
+        starts = torch.empty((num_seqs, width), dtype=torch.float32, device=zxg.device)
+        _run("mingru_scan_chunks", library().ts_mingru_scan_chunks(
+            _ptr(out), _code(out_dtype), _ptr(zxg), _code(zxg.dtype), _ptr(bias), 0 if bias is None else _code(bias.dtype),
+            _ptr(state), _ptr(folds), _ptr(starts), _ptr(cu_seqlens), _ptr(state_slots), num_seqs, width, longest, _stream()))
+        return out
     _run("mingru_scan", library().ts_mingru_scan(
         _ptr(out), _code(out_dtype), _ptr(zxg), _code(zxg.dtype), _ptr(bias), 0 if bias is None else _code(bias.dtype),
         _ptr(state), _ptr(cu_seqlens), _ptr(state_slots), num_seqs, width, mingru_waves(longest), _stream()))
