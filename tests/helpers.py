@@ -57,4 +57,8 @@ def rugezen_configs():
     Q = RugezenConfig(vocab=131, width=48, norm_eps=1e-4, residual_mult=1.0,
                       layers=(RugezenLayer("attention", att_q, 64), RugezenLayer("mingru", RugezenMinGRU(width=100), None),
                               RugezenLayer("mingru", RugezenMinGRU(width=16), 40), RugezenLayer("attention", att_s, 56)))
-    return {"P": (P, 3), "Q": (Q, 4)}
+    # sizes that are multiples of nothing in particular: no kernel's fast path takes them
+    att_t = RugezenAttention(heads=3, kv_heads=1, dim=20, vdim=12, rot_dims=6, rot_base=100.0, scale=0.3, softcap=5.0)
+    R = RugezenConfig(vocab=77, width=99, norm_eps=1e-5, residual_mult=0.8, loop_start=1, loop_stop=2, loop_times=2,
+                      layers=(RugezenLayer("attention", att_t, 52), RugezenLayer("mingru", RugezenMinGRU(width=35), 44)))
+    return {"P": (P, 3), "Q": (Q, 4), "R": (R, 5)}

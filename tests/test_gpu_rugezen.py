@@ -334,14 +334,14 @@ def test_attention_window_edges(dtype):
 
 # ---- whole models through trace replay ---------------------------------------------------------
 
-LENGTHS = {"P": [1, 2, 40, 150], "Q": [3, 66, 129, 200]}
+LENGTHS = {"P": [1, 2, 40, 150], "Q": [3, 66, 129, 200], "R": [1, 7, 65, 140]}
 # float32: only the engine's own 32-bit rounding separates it from the 64-bit oracle (worst seen 2.5e-7).
 # bfloat16: activations are rounded to 8 bits of mantissa at every projection's input; the worst logit was
 # off by 1.8e-3 in every way of feeding, the logits' spread being 0.16; the bound is under three times that.
 TOL = {"float32": dict(atol=3e-6, rtol=1e-5), "bfloat16": dict(atol=5e-3, rtol=0.0)}
 
 
-@pytest.fixture(scope="module", params=["P", "Q"])
+@pytest.fixture(scope="module", params=["P", "Q", "R"])
 def case(request, tmp_path_factory):
     from tinyserve_llm_amd.weights.random_init import write_random_model
     name = request.param

@@ -27,7 +27,7 @@ def test_round_trip_and_registry(tmp_path):
 
 
 def test_run_order_and_plans():
-    P, Q = (c for c, _ in rugezen_configs().values())
+    P, Q = (rugezen_configs()[k][0] for k in "PQ")
     assert P.run_order() == [0, 1, 0, 1, 0, 1, 2] and Q.run_order() == [0, 1, 2, 3]
     model = DecoderModel(__import__("tinyserve_llm_amd.models.rugezen", fromlist=["x"]).rugezen_spec(P))
     # every pass of the looped stretch has a cache or a state of its own

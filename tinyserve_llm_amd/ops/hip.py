@@ -1431,6 +1431,10 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
         return gemm_rows64(x, packed.by16, out_dtype)
     if _many_rows == "tiled" and tiled_takes(x, weight):
         return gemm_tiled(x, weight, out_dtype=out_dtype)
+    if x.shape[1] % 8 or x.stride(0) % 8 or weight.stride(0) % 8:
+        # rows that are no whole 16-byte pieces: the library has no algorithm for every such shape; the
+        # exact kernel takes any (32-bit multiply-adds, slower, for sizes no real model has)
+        return gemm_exact(x, weight, out_dtype)
     return gemm_library(x, weight, out_dtype)
 
 
