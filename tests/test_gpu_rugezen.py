@@ -523,3 +523,46 @@ def test_greedy_generation_through_the_scheduler(case):
             row = oracle.logits(ids)[-1]
             assert float(row.max() - row[tok]) <= 0.1, "a bfloat16 token far from the plain model's best"
             ids.append(tok)
+
+
+def test_forked_continuations_copy_state_and_pages(case):
+    """n = 3 at temperature 0: the continuations part after the prompt, each with a copy of the minGRU
+    state and the prompt's pages shared; all three must be the oracle's greedy continuation. And a pool
+    so small that requests are preempted and fed again from their first token (their state slot
+    starts from zero again)."""
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    name, folder, config, prompts, oracle, _ = case
+    p = prompt(11, 45, config.vocab)
+    want = oracle.greedy(p, 10)
+    sc = SchedulerConfig(max_model_len=128, max_num_seqs=4, max_num_batched_tokens=64, max_prefill_chunk=16)
+    llm = LLM(folder, sc, CacheConfig(block_size=16), dtype=torch.float32, num_blocks=24)
+    got = llm.generate([p], SamplingParams(max_tokens=10, temperature=0.0, n=3, ignore_eos=True))
+    assert got[0].token_ids == [want, want, want]
+    # four requests of 60 to 70 tokens that grow by 30 on 14 pages of 16: they do not all fit to the end
+    many = [prompt(20 + i, 60 + 3 * i, config.vocab) for i in range(4)]
+    wants = [oracle.greedy(q, 30) for q in many]
+    small = LLM(folder, sc, CacheConfig(block_size=16, caching=False), dtype=torch.float32, num_blocks=14)
+    out = small.generate(many, SamplingParams(max_tokens=30, temperature=0.0, ignore_eos=True))
+    assert [r.token_ids[0] for r in out] == wants
+    assert small.scheduler.stats().preemptions > 0, "the pool was meant to be too small"
+
+
+def test_command_line_generates_from_a_model_folder(case, tmp_path):
+    import json
+    import os
+    import subprocess
+    import sys
+    name, folder, config, prompts, oracle, _ = case
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = prompts[2]
+    out = tmp_path / "record.json"
+    cmd = [sys.executable, "-m", "tinyserve_llm_amd.generate", "--model", folder, "--prompt-ids", ",".join(map(str, p)),
+           "--max-tokens", "6", "--temperature", "0", "--ignore-eos", "--dtype", "float32", "--block-size", "32",
+           "--num-blocks", "16", "--max-model-len", "256", "--max-num-seqs", "4", "--out", str(out)]
+    r = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    record = json.loads(out.read_text())
+    text = json.dumps(record)
+    assert json.dumps(oracle.greedy(p, 6)).replace(" ", "") in text.replace(" ", ""), text[:500]
