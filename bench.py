@@ -170,10 +170,10 @@ def designs(args) -> int:
     hidden, nh, nkv, hd, inter, vocab = (sh["hidden_size"], sh["num_attention_heads"], sh["num_key_value_heads"], sh["head_dim"],
                                          sh["intermediate_size"], sh["vocab_size"])
     llama = LlamaConfig(num_hidden_layers=layers, rope_scaling=RopeScaling(**{**ROPE, "factor": sizes["rope_factor"]}), **sh)
-    att = RugezenAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, rot_dims=hd // 2, rot_base=sh["rope_theta"], scale=hd ** -0.5,
-                           softcap=50.0)
+    att = RugezenAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, rot_dims=hd // 2, rot_base=1.0e6, scale=hd ** -0.5,
+                           softcap=30.0)
     ff = 3 * inter // 2                  # two matrices of this width hold what the gated feed-forward's three hold
-    rug = RugezenConfig(vocab=vocab, width=hidden, norm_eps=1e-5, residual_mult=0.5, layers=tuple(
+    rug = RugezenConfig(vocab=vocab, width=hidden, norm_eps=1e-6, residual_mult=0.6, layers=tuple(
         RugezenLayer("mingru", RugezenMinGRU(width=hidden), ff) if i % 4 == 2 else RugezenLayer("attention", att, ff)
         for i in range(layers)))
     prompt_len = args.context
@@ -287,7 +287,7 @@ def designs(args) -> int:
             flops = 4 * nh * hd * keys
             nbytes = sum(s0 + n for s0, n in zip(starts, counts)) * 2 * nkv * hd * 2
             plain_us = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5))
-            general_us = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5, softcap=50.0, sink=True))
+            general_us = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5, softcap=30.0, sink=True))
             if T > 64:
                 pairs[f"attention, {label}"] = {"llama_us": plain_us, "rugezen_us": general_us, "flops": flops,
                                                 "llama_frac_of_mfma": flops / plain_us * 1e6 / mfma_peak,
@@ -312,7 +312,7 @@ def designs(args) -> int:
             w16 = torch.ones(hidden, device="cuda").to(bf)
             x32, a32, b32 = (torch.randn(T, hidden, device="cuda") for _ in range(3))
             us_a = timed(lambda: hip.rmsnorm(x16, w16, 1e-5, r16))
-            us_b = timed(lambda: hip.stream_update_norm(x32, a32, b32, w16, 0.5, (w16, w16), 1e-5, out_dtype=bf))
+            us_b = timed(lambda: hip.stream_update_norm(x32, a32, b32, w16, 0.6, (w16, w16), 1e-6, out_dtype=bf))
             bytes_a, bytes_b = T * hidden * 2 * 4, T * hidden * (4 * 4 + 2 * 2)
             pairs[f"residual sum and norms, {label}"] = {"llama_us": us_a, "rugezen_us": us_b, "llama_bytes": bytes_a, "rugezen_bytes": bytes_b,
                                                          "llama_frac_of_read": bytes_a / us_a * 1e6 / read_peak,

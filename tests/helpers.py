@@ -61,4 +61,9 @@ def rugezen_configs():
     att_t = RugezenAttention(heads=3, kv_heads=1, dim=20, vdim=12, rot_dims=6, rot_base=100.0, scale=0.3, softcap=5.0)
     R = RugezenConfig(vocab=77, width=99, norm_eps=1e-5, residual_mult=0.8, loop_start=1, loop_stop=2, loop_times=2,
                       layers=(RugezenLayer("attention", att_t, 52), RugezenLayer("mingru", RugezenMinGRU(width=35), 44)))
-    return {"P": (P, 3), "Q": (Q, 4), "R": (R, 5)}
+    # a width that the weight-streaming kernels take (steps of few rows then run the fused forms), heads of a
+    # matrix-core size
+    att_u = RugezenAttention(heads=8, kv_heads=2, dim=64, vdim=64, rot_dims=64, rot_base=20000.0, scale=0.11, softcap=8.0)
+    S = RugezenConfig(vocab=300, width=512, norm_eps=1e-6, residual_mult=0.45, loop_start=0, loop_stop=1, loop_times=2,
+                      layers=(RugezenLayer("attention", att_u, 640), RugezenLayer("mingru", RugezenMinGRU(width=256), 768)))
+    return {"P": (P, 3), "Q": (Q, 4), "R": (R, 5), "S": (S, 6)}

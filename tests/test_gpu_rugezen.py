@@ -224,7 +224,7 @@ def attention_case(dtype, H, G, D, V, page, length, queries, stand_out, scale, s
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(4, 2, 32, 48), (2, 2, 16, 16), (6, 1, 24, 8), (4, 1, 96, 96)])
+@pytest.mark.parametrize("sizes", [(4, 2, 32, 48), (2, 2, 16, 16), (6, 1, 24, 8), (6, 2, 96, 96)])
 def test_attention_far_keys_page_borders_and_first_tokens(dtype, sizes):
     H, G, D, V = sizes
     page, length = 16, 700
@@ -261,7 +261,7 @@ def step_context(table, page, starts, counts):
                        page_size=page), positions
 
 
-@pytest.mark.parametrize("sizes", [(4, 1, 96, 96), (8, 2, 64, 64), (2, 2, 128, 128), (4, 4, 32, 32), (16, 1, 64, 64)])
+@pytest.mark.parametrize("sizes", [(6, 3, 96, 96), (8, 2, 64, 64), (2, 2, 128, 128), (4, 4, 32, 32), (16, 1, 64, 64)])
 @pytest.mark.parametrize("cap, sink", [(30.0, True), (0.0, True), (0.8, False)])
 def test_matrix_core_kernels_general_variants(sizes, cap, sink):
     """bfloat16 heads of the matrix-core kernels' sizes go to those kernels' general variants: single
@@ -310,10 +310,10 @@ def test_matrix_core_kernels_general_variants(sizes, cap, sink):
 
 def test_the_sink_weighs_most_on_the_first_tokens():
     """One visible key of score s: the weight is e^s / (1 + e^s), not 1."""
-    out, want, v = attention_case(torch.float32, 2, 1, 16, 16, 16, 3, [0], {}, 0.25, 50.0, True)
+    out, want, v = attention_case(torch.float32, 2, 1, 16, 16, 16, 3, [0], {}, 0.25, 40.0, True)
     torch.testing.assert_close(out, want, atol=1e-6, rtol=1e-5)
     assert float((out[0, 0] / v[0, 0]).mean()) < 0.9
-    no_sink, _, _ = attention_case(torch.float32, 2, 1, 16, 16, 16, 3, [0], {}, 0.25, 50.0, False)
+    no_sink, _, _ = attention_case(torch.float32, 2, 1, 16, 16, 16, 3, [0], {}, 0.25, 40.0, False)
     torch.testing.assert_close(no_sink[0, 0], v[0, 0], atol=1e-6, rtol=1e-5)
 
 
@@ -334,14 +334,15 @@ def test_attention_window_edges(dtype):
 
 # ---- whole models through trace replay ---------------------------------------------------------
 
-LENGTHS = {"P": [1, 2, 40, 150], "Q": [3, 66, 129, 200], "R": [1, 7, 65, 140]}
-# float32: only the engine's own 32-bit rounding separates it from the 64-bit oracle (worst seen 2.5e-7).
-# bfloat16: activations are rounded to 8 bits of mantissa at every projection's input; the worst logit was
-# off by 1.8e-3 in every way of feeding, the logits' spread being 0.16; the bound is under three times that.
-TOL = {"float32": dict(atol=3e-6, rtol=1e-5), "bfloat16": dict(atol=5e-3, rtol=0.0)}
+LENGTHS = {"P": [1, 2, 40, 150], "Q": [3, 66, 129, 200], "R": [1, 7, 65, 140], "S": [2, 33, 64, 130]}
+# Bounds on a logit's error as a share of the logits' spread (their standard deviation over the oracle's rows).
+# float32: only the engine's own 32-bit rounding separates it from the 64-bit oracle (worst seen 4e-6 of the spread).
+# bfloat16: activations are rounded to 8 bits of mantissa at every projection's input; the worst logit was off by
+# 1.5 % of the spread in every way of feeding; the bound is twice that.
+TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 
 
-@pytest.fixture(scope="module", params=["P", "Q", "R"])
+@pytest.fixture(scope="module", params=["P", "Q", "R", "S"])
 def case(request, tmp_path_factory):
     from tinyserve_llm_amd.weights.random_init import write_random_model
     name = request.param
@@ -360,13 +361,14 @@ def replayer(folder, dtype, max_tokens):
 
 def check(got, oracle_rows, dtype):
     assert got, "nothing was compared"
+    spread = float(torch.cat([o.flatten() for o in oracle_rows]).std())
     worst = 0.0
     for (r, pos), row in got.items():
         want = oracle_rows[r][pos]
-        torch.testing.assert_close(row.double().cpu(), want, **TOL[dtype], msg=lambda m: f"request {r} position {pos}: {m}")
+        torch.testing.assert_close(row.double().cpu(), want, atol=TOL[dtype] * spread, rtol=0.0,
+                                   msg=lambda m: f"request {r} position {pos}: {m}")
         worst = max(worst, float((row.double().cpu() - want).abs().max()))
-    spread = float(torch.cat([o.flatten() for o in oracle_rows]).std())
-    print(f"[{dtype}] worst absolute logit error {worst:.3e} over {len(got)} rows (the logits' spread is {spread:.2f})")
+    print(f"[{dtype}] worst logit error {worst / spread:.3e} of the logits' spread ({spread:.2f}) over {len(got)} rows")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -566,3 +568,23 @@ def test_command_line_generates_from_a_model_folder(case, tmp_path):
     record = json.loads(out.read_text())
     text = json.dumps(record)
     assert json.dumps(oracle.greedy(p, 6)).replace(" ", "") in text.replace(" ", ""), text[:500]
+
+
+@pytest.mark.parametrize("rows", [1, 3, 8])
+@pytest.mark.parametrize("activation", ["relu2", "gelu_tanh", "silu"])
+def test_projection_with_bias_and_activation_on_the_way_out(rows, activation):
+    """Few rows: the up projection's kernel applies bias and activation to its 32-bit sums itself."""
+    h = hip()
+    K, N = 512, 328
+    x, x64 = rounded(torch.randn(rows, K), torch.bfloat16)
+    w, w64 = rounded(torch.randn(N, K) * 0.05, torch.bfloat16)
+    b, b64 = rounded(torch.randn(N), torch.bfloat16)
+    assert h.skinny8_act_takes(x, w, b)
+    fn = {"relu2": plain.squared_relu, "gelu_tanh": plain.gelu_tanh, "silu": lambda v: v * torch.sigmoid(v)}[activation]
+    want = fn(x64 @ w64.T + b64)
+    got32 = h.gemm_skinny8_act(x, w, b, activation, torch.float32)
+    torch.testing.assert_close(got32.cpu().to(F64), want, atol=2e-5, rtol=2e-5)
+    got16 = h.gemm_skinny8_act(x, w, b, activation, torch.bfloat16, h.pack_weight8(w))
+    torch.testing.assert_close(got16.cpu().to(F64), want, atol=2e-2, rtol=1e-2)
+    none = h.gemm_skinny8_act(x, w, None, activation, torch.float32)
+    torch.testing.assert_close(none.cpu().to(F64), fn(x64 @ w64.T), atol=2e-5, rtol=2e-5)

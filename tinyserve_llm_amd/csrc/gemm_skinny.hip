@@ -918,6 +918,16 @@ gemm_skinny8_kernel(const SkinnyArgs a) {
   for (int wv = 0; wv < nwaves; ++wv)                    // waves in order, within a wave the lower half of k first
     sum += smem[wv * 256 + m * 16 + nl] + smem[wv * 256 + (m + 8) * 16 + nl + 8];
   const int n = n0 + nl;
+  if constexpr (!NEXT) {
+    // an activation on the way out, act(sum + bias[n]), for a feed-forward without a gate: its code travels in
+    // ssq_parts and its bias in nw, which this form leaves unused otherwise (1: relu squared, 2: gelu, tanh form, 3: silu)
+    if (a.ssq_parts) {
+      const float z = sum + (a.nw && n < a.N ? bf2f(a.nw[n]) : 0.f);
+      if (a.ssq_parts == 1) { const float p = fmaxf(z, 0.f); sum = p * p; }
+      else if (a.ssq_parts == 2) sum = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+      else sum = z / (1.0f + expf(-z));
+    }
+  }
   if constexpr (NEXT) {
     // EPI_NEXT (see the top of the file): the eight threads of a row hold the tile's eight columns
     const bool in = m < a.M && n < a.N;
@@ -1025,6 +1035,25 @@ extern "C" int ts_gemm_skinny8_bf16(void* y, const void* x, const void* w, int M
     return sk8_dispatch<bf16_t, true>(a, stream);
   }
   if (!y || ldy < N) return TS_BAD_SHAPE;
+  if (out_dtype == 1) return sk8_dispatch<bf16_t>(a, stream);
+  if (out_dtype == 0) return sk8_dispatch<float>(a, stream);
+  return TS_BAD_DTYPE;
+}
+
+// The same product with act(. + bias) on the way out (act 1: relu squared, 2: gelu in its tanh form, 3: silu; bias
+// bfloat16 [N] or null): the up projection of a feed-forward without a gate, for steps of few rows.
+extern "C" int ts_gemm_skinny8_act_bf16(void* y, const void* x, const void* w, int M, int N, int K, int64_t ldx, int64_t ldw,
+                                        int64_t ldy, int out_dtype, int packed, const void* bias, int act, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return TS_OK;
+  if (M > 8 || K <= 0 || ldx % 8 || ldx < K || (!packed && (ldw % 8 || ldw < K)) || (packed && N % 8) || act < 1 || act > 3)
+    return TS_BAD_SHAPE;
+  if (((uintptr_t)x | (uintptr_t)w) & 15) return TS_BAD_SHAPE;
+  if (!y || ldy < N) return TS_BAD_SHAPE;
+  SkinnyArgs a = {};
+  a.x = (const bf16_t*)x; a.w = (const bf16_t*)w; a.y = y; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy;
+  a.packed = packed;
+  a.nw = (const bf16_t*)bias;
+  a.ssq_parts = act;
   if (out_dtype == 1) return sk8_dispatch<bf16_t>(a, stream);
   if (out_dtype == 0) return sk8_dispatch<float>(a, stream);
   return TS_BAD_DTYPE;

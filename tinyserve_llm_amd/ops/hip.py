@@ -70,6 +70,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_paged_attention_prefill": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i, i, i, p, p, i, p],
         "ts_gemm_skinny_bf16": [p, p, p, p, p, p, i, i, i, i64, i64, i64, f, i, i, i, i, p, i, p, p, p, p, p, i, p],
         "ts_gemm_skinny8_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, p, p, p, p, i, p, p, p, i, i, i, i, p],
+        "ts_gemm_skinny8_act_bf16": [p, p, p, i, i, i, i64, i64, i64, i, i, p, i, p],
         "ts_gemm_rows64_bf16": [p, p, p, i, i, i, i64, i64, i, i, p, i, f, p],
         "ts_gemm_rows64_sliced_bf16": [p, p, p, p, i, i, i, i64, i, p, p, p, p, p, i64, p],
         "ts_gemm_rows64_sliced_rope_bf16": [p, p, p, p, i, i, i64, i, p, i, f, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64,
@@ -989,6 +990,36 @@ def gemm_skinny8(x: "torch.Tensor | PackedRows8 | SplitAttention", weight: torch
     _run("gemm_skinny8", library().ts_gemm_skinny8_bf16(
         _ptr(out), x_arg, _ptr(weight if packed8 is None else packed8), M, N, K, ldx, weight.stride(0),
         out.stride(0), _code(out_dtype), int(packed8 is not None), None, None, None, None, None, int(x_packed), *comb, _stream()))
+    return out
+
+
+def skinny8_act_takes(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None) -> bool:
+    """Whether `gemm_skinny8_act` serves these operands: the 8-row form's shapes, bfloat16 throughout."""
+    return (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2 and weight.dim() == 2
+            and (bias is None or (bias.dtype == torch.bfloat16 and bias.is_contiguous()))
+            and skinny8_takes(x.shape[0], weight.shape[0], weight.shape[1]) and _dense_rows(x) and weight.is_contiguous()
+            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def gemm_skinny8_act(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, activation: str,
+                     out_dtype: torch.dtype = torch.bfloat16, packed8: torch.Tensor | None = None) -> torch.Tensor:
+    """act(x · weight^T + bias) for up to 8 rows of x by the weight-streaming kernel's 8-row form, the bias
+    and the activation (one of `ACTIVATIONS` but "none") applied to the 32-bit sums on their way out."""
+    _gpu(x, weight, bias, packed8)
+    _need(skinny8_act_takes(x, weight, bias), "gemm_skinny8_act: the 8-row form's shapes, bfloat16, dense aligned rows")
+    _need(activation in ACTIVATIONS and activation != "none", lambda: f"activation {activation!r}")
+    _need(bias is None or bias.shape == (weight.shape[0],), "the bias must be [N]")
+    M, K = x.shape
+    N = weight.shape[0]
+    if packed8 is not None:
+        steps = skinny8_steps(K)
+        _need(packed8.dtype == torch.bfloat16 and packed8.shape == (-(-N // 8), K // (64 * steps), steps, 64, 8)
+              and packed8.is_contiguous() and packed8.data_ptr() % 16 == 0 and N % 8 == 0,
+              lambda: f"the packed copy does not belong to a weight of {N} x {K}")
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _run("gemm_skinny8_act", library().ts_gemm_skinny8_act_bf16(
+        _ptr(out), _ptr(x), _ptr(weight if packed8 is None else packed8), M, N, K, x.stride(0), weight.stride(0), out.stride(0),
+        _code(out_dtype), int(packed8 is not None), _ptr(bias), ACTIVATIONS[activation], _stream()))
     return out
 
 

@@ -43,7 +43,7 @@ class GatedMLP(FeedForward):
 class DenseMLP(FeedForward):
     """A feed-forward without a gate: W_down act(W_up h + b_up) + b_down, `activation` one of
     `hip.ACTIVATIONS` ("relu2": the square of relu). The up projection's sums stay 32-bit until bias and
-    activation are applied; the down projection's result is 32-bit. `forward(..., defer_bias=True)`
+    activation are applied (by the projection's own kernel for steps of few rows, by a kernel of their own otherwise); the down projection's result is 32-bit. `forward(..., defer_bias=True)`
     returns (W_down a, b_down) for a caller that adds the bias with its residual sum."""
 
     graph_safe = True
@@ -73,8 +73,13 @@ class DenseMLP(FeedForward):
         return sum(c.nbytes() for c in (self.up_packed, self.down_packed) if c is not None)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, defer_bias: bool = False):
-        up = linear(x, self.up, out_dtype=torch.float32, packed=self.up_packed)
-        act = hip.bias_activation(up, self.up_bias, self.activation, x.dtype)
+        if hip.skinny8_act_takes(x, self.up, self.up_bias):
+            # few rows: bias and activation ride on the projection's way out, from its 32-bit sums
+            act = hip.gemm_skinny8_act(x, self.up, self.up_bias, self.activation, x.dtype,
+                                       None if self.up_packed is None else self.up_packed.by8)
+        else:
+            up = linear(x, self.up, out_dtype=torch.float32, packed=self.up_packed)
+            act = hip.bias_activation(up, self.up_bias, self.activation, x.dtype)
         down = linear(act, self.down, out_dtype=torch.float32, packed=self.down_packed)
         if defer_bias:
             return down, self.down_bias
