@@ -338,8 +338,8 @@ LENGTHS = {"P": [1, 2, 40, 150], "Q": [3, 66, 129, 200], "R": [1, 7, 65, 140], "
 # Bounds on a logit's error as a share of the logits' spread (their standard deviation over the oracle's rows).
 # float32: only the engine's own 32-bit rounding separates it from the 64-bit oracle (worst seen 4e-6 of the spread).
 # bfloat16: activations are rounded to 8 bits of mantissa at every projection's input; the worst logit was off by
-# 1.5 % of the spread in every way of feeding; the bound is twice that.
-TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+# 1.2 to 2.6 % of the spread, configuration by configuration, in every way of feeding; the bound is twice the largest.
+TOL = {"float32": 2e-5, "bfloat16": 5e-2}
 
 
 @pytest.fixture(scope="module", params=["P", "Q", "R", "S"])

@@ -64,8 +64,8 @@ class DenseMLP(FeedForward):
         specs = {"up": ParamSpec((self.intermediate_size, self.hidden_size)),
                  "down": ParamSpec((self.hidden_size, self.intermediate_size))}
         if self.has_bias:
-            specs["up_bias"] = ParamSpec((self.intermediate_size,), init=(0.0, 0.1))
-            specs["down_bias"] = ParamSpec((self.hidden_size,), init=(0.0, 0.1))
+            specs["up_bias"] = ParamSpec((self.intermediate_size,), init=(0.0, 0.02))
+            specs["down_bias"] = ParamSpec((self.hidden_size,), init=(0.0, 0.02))
         return specs
 
     def keep_streaming_copies(self) -> int:
