@@ -91,10 +91,10 @@ qkv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restri
 
 // The same for heads whose sizes are multiples of eight: a thread holds a piece of eight consecutive elements
 // of a head (whole pairs of the interleaved layout; for the halves layout the partner piece is fetched as well), GS threads side by side hold a head (GS the power of two that covers the larger head size),
-// and a thread takes every `slices`-th head of its token: 8 slices for steps of many tokens, so that a token's
-// angles are taken 8 times and not once per head; a slice per head for steps of few, which have threads to spare
+// and a thread takes every `slices`-th head of its token: 16 slices for steps of many tokens, so that a token's
+// angles are taken 16 times and not once per head; a slice per head for steps of few, which have threads to spare
 // and no time for one head after the other. All of a thread's loads for a head go out together.
-#define AG_SLICES 8
+#define AG_SLICES 16
 template <typename T> struct Piece8;
 template <> struct Piece8<float> {
   static __device__ __forceinline__ void ld(const float* p, float* o) {
@@ -144,29 +144,37 @@ qkv_finish_pieces_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* _
   const int page = stores ? slot / page_size : 0, off = stores ? slot - page * page_size : 0;
   // this piece's angles: element e turns with pair (d0 + e) / 2 (interleaved) or (d0 + e) mod half (halves)
   float cs[8], sn[8];
+  auto angles = [&]() {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    cs[e] = 1.f; sn[e] = 0.f;
-    const int d = d0 + e;
-    if (d < rot && (!interleaved || !(e & 1))) {
-      const int pair = interleaved ? d >> 1 : (d < half ? d : d - half);
-      const double angle = (double)pos * freqs[pair];
-      const double turns = rint(angle * 0.15915494309189535);
-      sincosf((float)fma(-turns, 6.283185307179586, angle), &sn[e], &cs[e]);
+    for (int e = 0; e < 8; ++e) {
+      cs[e] = 1.f; sn[e] = 0.f;
+      const int d = d0 + e;
+      if (d < rot && (!interleaved || !(e & 1))) {
+        const int pair = interleaved ? d >> 1 : (d < half ? d : d - half);
+        // the angle in 64-bit, brought to [-pi, pi] before the 32-bit sine and cosine
+        const double angle = (double)pos * freqs[pair];
+        const double turns = rint(angle * 0.15915494309189535);
+        sincosf((float)fma(-turns, 6.283185307179586, angle), &sn[e], &cs[e]);
+      }
+      if (interleaved && (e & 1)) { cs[e] = cs[e - 1]; sn[e] = sn[e - 1]; }
     }
-    if (interleaved && (e & 1)) { cs[e] = cs[e - 1]; sn[e] = sn[e - 1]; }
-  }
+  };
   const int64_t row = (int64_t)(nh + nkv) * hd + (int64_t)nkv * vd_size;
   const TI* trow = qkv + (int64_t)t * row;
-  for (int h = slice; h < heads; h += slices) {
+  // where a head's piece lies in the token's row, and how many of its elements there are for this thread (8 or 0)
+  auto piece_of = [&](int h) {
+    const bool is_v = h >= nh + nkv;
+    return trow + (is_v ? (int64_t)(nh + nkv) * hd + (int64_t)(h - nh - nkv) * vd_size : (int64_t)h * hd) + d0;
+  };
+  auto has_piece = [&](int h) { return h < heads && d0 < (h >= nh + nkv ? vd_size : hd); };
+  // everything after a head's piece has arrived
+  auto finish = [&](int h, const float (&x)[8]) {
     const bool is_q = h < nh, is_v = h >= nh + nkv;
     const int size = is_v ? vd_size : hd;
     const bool mine = d0 < size;
-    const TI* src = trow + (is_v ? (int64_t)(nh + nkv) * hd + (int64_t)(h - nh - nkv) * vd_size : (int64_t)h * hd);
-    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, w[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (mine) Piece8<TI>::ld(src + d0, x);
+    float w[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const bool turns_here = !is_v && mine && d0 < rot;
-    if (turns_here && !interleaved) Piece8<TI>::ld(src + (d0 < half ? d0 + half : d0 - half), w);   // (rot a multiple of 16: whole pieces)
+    if (turns_here && !interleaved) Piece8<TI>::ld(piece_of(h) + (d0 < half ? half : -half), w);   // (rot a multiple of 16: whole pieces)
     float y[8], squares = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -180,22 +188,46 @@ qkv_finish_pieces_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* _
       squares = fmaf(v, v, squares);
     }
     float scale = 1.0f;
-    if (is_v ? v_norm : qk_norm) {                           // (uniform: every lane of the wave shuffles)
+    if (is_v ? v_norm : qk_norm) {                           // (the same for all threads of a head: they shuffle together)
 #pragma unroll
       for (int o = GS / 2; o > 0; o >>= 1) squares += __shfl_xor(squares, o, TS_WAVE);
       scale = 1.0f / sqrtf(squares / (float)size + (is_v ? v_eps : qk_eps));
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) y[e] *= scale;
-    if (!mine || !live) continue;
+    if (!mine || !live) return;
     if (is_q) Piece8<TO>::st(q_out + ((int64_t)t * nh + h) * hd + d0, y);
-    else if (!stores) continue;
+    else if (!stores) return;
     else if (!is_v) Piece8<TO>::st(k_cache + page * kp + off * ks + (int64_t)(h - nh) * kh + d0, y);
     else {
       TO* dst = v_cache + page * vp + off * vs + (int64_t)(h - nh - nkv) * vh + (int64_t)d0 * vd;
 #pragma unroll
       for (int e = 0; e < 8; ++e) Num<TO>::st(dst + (int64_t)e * vd, y[e]);
     }
+  };
+  constexpr int AHEAD = 8;                                   // heads whose pieces a thread asks for before it works on the first
+  if ((heads + slices - 1) / slices <= AHEAD) {
+    float xs[AHEAD][8];
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) {
+      const int h = slice + k * slices;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xs[k][e] = 0.f;
+      if (has_piece(h)) Piece8<TI>::ld(piece_of(h), xs[k]);
+    }
+    angles();                                                // (while the pieces are on their way)
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) {
+      const int h = slice + k * slices;
+      if (h < heads) finish(h, xs[k]);
+    }
+    return;
+  }
+  angles();
+  for (int h = slice; h < heads; h += slices) {
+    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (has_piece(h)) Piece8<TI>::ld(piece_of(h), x);
+    finish(h, x);
   }
 }
 
@@ -216,7 +248,7 @@ v_finish_kernel(TO* __restrict__ v_cache, const TI* __restrict__ qkv, const int3
   const int nt = min(AG_VTOK, num_tokens - t0);
   // the tile's rows into LDS, every thread's loads independent of each other
   const TI* tile = qkv + (int64_t)t0 * row + v_first + (int64_t)g * vd_size;
-#pragma unroll 4
+#pragma unroll 8
   for (int i = threadIdx.x; i < nt * vd_size; i += AG_WAVES * TS_WAVE) {
     const int tl = i / vd_size, d = i - tl * vd_size;
     rows_s[tl][d] = Num<TI>::ld(tile + (int64_t)tl * row + d);
