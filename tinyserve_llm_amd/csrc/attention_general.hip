@@ -8,7 +8,10 @@
 //     differ in size.
 //   * `ts_paged_attention_general`: one wavefront per (token, query head) over the request's pages, causal,
 //     optionally windowed; score = q.k * scale, optionally capped as cap * tanh(score / cap); softmax,
-//     optionally with a sink: a key of score 0 that has no value, i.e. one more in the denominator.
+//     optionally with a sink: a key of score 0 that has no value, i.e. one more in the denominator; or with
+//     learned sinks, exp(sinks[head]) in the denominator instead of 1. Optionally a penalty on distance,
+//     slopes[head] * (position - key's position), is taken off every score, and the output row is multiplied
+//     element by element by sigmoid(gate) on its way out (gate: 32-bit rows of the step, one element per output).
 //     Scores, weights and the weighted sum are 32-bit. Keys are visited in chunks of 64 counted from position
 //     0, so the order of every sum depends on the token's position alone.
 #include "common.h"
@@ -324,7 +327,8 @@ paged_attention_general_kernel(T* __restrict__ out, const T* __restrict__ q, con
                                const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
                                int num_tokens, int nh, int nkv, int hd, int vd_size, int page_size, int64_t kp, int64_t ks,
                                int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int max_blocks, float scale,
-                               float softcap, int sink, int window, int page_run) {
+                               float softcap, int sink, int window, int page_run, const float* __restrict__ sinks,
+                               const float* __restrict__ slopes, const float* __restrict__ gate, int64_t gate_stride) {
   __shared__ float q_s[AG_WAVES][AG_MAX_HD];
   __shared__ float p_s[AG_WAVES][TS_WAVE];
   __shared__ int64_t row_s[AG_WAVES][TS_WAVE];   // element offset of each key's value row
@@ -341,7 +345,9 @@ paged_attention_general_kernel(T* __restrict__ out, const T* __restrict__ q, con
 
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   // the sink is a key of score 0 without a value: it starts the running maximum and the sum
-  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  // (a learned sink is the same key with a score of its own)
+  float m = sinks ? sinks[h] : sink ? 0.f : -INFINITY, l = (sinks || sink) ? 1.f : 0.f;
+  const float slope = slopes ? slopes[h] : 0.f;
   float acc[AG_MAX_HD / TS_WAVE] = {0.f, 0.f, 0.f, 0.f};
   const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
 
@@ -359,6 +365,7 @@ paged_attention_general_kernel(T* __restrict__ out, const T* __restrict__ q, con
       for (int d = 0; d < hd; ++d) dot = fmaf(q_s[wave][d], Num<T>::ld(kr + d), dot);
       s = dot * scale;
       if (softcap > 0.f) s = softcap * tanhf(s * inv_cap);
+      s -= slope * (float)(pos - key);
     }
     const float m_new = fmaxf(m, wave_max(s));  // finite: the chunk holds at least one visible key
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -386,7 +393,11 @@ paged_attention_general_kernel(T* __restrict__ out, const T* __restrict__ q, con
 #pragma unroll
   for (int i = 0; i < AG_MAX_HD / TS_WAVE; ++i) {
     const int d = lane + i * TS_WAVE;
-    if (d < vd_size) Num<T>::st(orow + d, acc[i] * inv);
+    if (d < vd_size) {
+      float o = acc[i] * inv;
+      if (gate) o = o / (1.0f + expf(-gate[(int64_t)t * gate_stride + (int64_t)h * vd_size + d]));
+      Num<T>::st(orow + d, o);
+    }
   }
 }
 
@@ -395,7 +406,8 @@ extern "C" int ts_paged_attention_general(void* out, const void* q, const void* 
                                           const int32_t* positions, int num_tokens, int nh, int nkv, int hd, int vd_size,
                                           int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs,
                                           int64_t vh, int64_t vd, int max_blocks, float scale, float softcap, int sink,
-                                          int window, int dtype, int page_run, hipStream_t stream) {
+                                          int window, int dtype, int page_run, const float* sinks, const float* slopes,
+                                          const float* gate, int64_t gate_stride, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (hd <= 0 || hd > AG_MAX_HD || vd_size <= 0 || vd_size > AG_MAX_HD || nkv <= 0 || nh % nkv || page_size <= 0 ||
       max_blocks <= 0 || page_run < 0 || page_run > 16 || softcap < 0.f)
@@ -408,12 +420,12 @@ extern "C" int ts_paged_attention_general(void* out, const void* q, const void* 
     paged_attention_general_kernel<float><<<grid, block, 0, stream>>>(
         (float*)out, (const float*)q, (const float*)k_cache, (const float*)v_cache, block_tables, seq_of_token, positions,
         num_tokens, nh, nkv, hd, vd_size, page_size, kp, ks, kh, vp, vs, vh, vd, max_blocks, scale, softcap, sink, window,
-        page_run);
+        page_run, sinks, slopes, gate, gate_stride);
   else if (dtype == 1)
     paged_attention_general_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, seq_of_token, positions,
         num_tokens, nh, nkv, hd, vd_size, page_size, kp, ks, kh, vp, vs, vh, vd, max_blocks, scale, softcap, sink, window,
-        page_run);
+        page_run, sinks, slopes, gate, gate_stride);
   else
     return TS_BAD_DTYPE;
   return ts_check_launch();

@@ -1,0 +1,266 @@
+// A mixture of experts: every token goes through `top` of `experts` small gated feed-forward layers.
+//   * `ts_moe_route`: router logits z = W_r h in 32-bit (h as it is stored), scores s = sigmoid(z); the `top`
+//     experts with the largest s + correction are chosen (ties: the lower index); their weights are their s,
+//     divided by the chosen ones' sum (+ 1e-20) if `normalize`, times `scale`.
+//   * `ts_moe_group`: the step's (token, choice) pairs grouped by expert, and the groups cut into tiles of rows
+//     that one workgroup of the product takes: [expert, first index, rows] per tile, rows 0 for the tiles of the
+//     launch that the step does not fill (the launch is sized for the worst case, so nothing comes back to the host).
+//   * `ts_moe_gemm`: for every tile, rows of the operand (a token's row, or a pair's) times the tile's expert's
+//     matrix; with `glu` the matrix holds gate rows, then up rows, and the capped gated unit
+//     g = min(gate, L), u = clamp(up, -L, L), y = g sigmoid(slope g) (u + shift) leaves instead of the sums.
+//     Every row's sums run over k in ascending order whatever the tile it lands in.
+//   * `ts_moe_combine`: out[token] = sum over its choices, in order, of weight * the pair's row (+ a shared
+//     expert's row).
+// float32 runs 32-bit multiply-adds; bfloat16 operands go through the matrix cores with 32-bit sums.
+#include "common.h"
+
+#define MOE_THREADS 256
+#define MOE_ROUTE_TOKENS 4
+#define MOE_MAX_EXPERTS 1024
+#define MOE_MAX_TOP 32
+
+template <typename TX>
+__global__ void __launch_bounds__(MOE_THREADS)
+moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const TX* __restrict__ x,
+                 const float* __restrict__ router, const float* __restrict__ correction, int num_tokens, int K, int E, int top,
+                 float scale, int normalize) {
+  extern __shared__ float lds[];
+  float* s_s = lds;                                       // [MOE_ROUTE_TOKENS][E] scores
+  float* c_s = lds + MOE_ROUTE_TOKENS * E;                // [MOE_ROUTE_TOKENS][E] choice scores
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
+  const int t0 = blockIdx.x * MOE_ROUTE_TOKENS;
+  const int nt = min(MOE_ROUTE_TOKENS, num_tokens - t0);
+  for (int e = wave; e < E; e += MOE_THREADS / TS_WAVE) {
+    float acc[MOE_ROUTE_TOKENS];
+#pragma unroll
+    for (int r = 0; r < MOE_ROUTE_TOKENS; ++r) acc[r] = 0.f;
+    const float* wr = router + (int64_t)e * K;
+    for (int k = lane; k < K; k += TS_WAVE) {
+      const float w = wr[k];
+#pragma unroll
+      for (int r = 0; r < MOE_ROUTE_TOKENS; ++r)
+        if (r < nt) acc[r] = fmaf(w, Num<TX>::ld(x + (int64_t)(t0 + r) * K + k), acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < MOE_ROUTE_TOKENS; ++r) {
+      const float z = wave_sum(acc[r]);
+      if (lane == 0) {
+        const float s = 1.0f / (1.0f + expf(-z));
+        s_s[r * E + e] = s;
+        c_s[r * E + e] = s + (correction ? correction[e] : 0.f);
+      }
+    }
+  }
+  __syncthreads();
+  if (wave >= nt) return;                                 // a wave per token from here on
+  const int r = wave, t = t0 + wave;
+  float total = 0.f;
+  float picked[MOE_MAX_TOP];
+  int chosen[MOE_MAX_TOP];
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += TS_WAVE) {
+      const float c = c_s[r * E + e];
+      if (c > best) { best = c; at = e; }                 // (ascending e: the lower index wins a tie)
+    }
+#pragma unroll
+    for (int off = TS_WAVE / 2; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, TS_WAVE);
+      const int oa = __shfl_xor(at, off, TS_WAVE);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    if (at >= E) at = j;                                  // (scores that are no numbers: still valid indices)
+    chosen[j] = at;
+    picked[j] = s_s[r * E + at];
+    total += picked[j];
+    wave_sync();
+    if (lane == 0) c_s[r * E + at] = -INFINITY;
+    wave_sync();
+  }
+  const float mult = (normalize ? 1.0f / (total + 1e-20f) : 1.0f) * scale;
+  if (lane == 0)
+    for (int j = 0; j < top; ++j) {
+      ids_out[(int64_t)t * top + j] = chosen[j];
+      w_out[(int64_t)t * top + j] = picked[j] * mult;
+    }
+}
+
+extern "C" int ts_moe_route(int32_t* ids_out, float* w_out, const void* x, int x_dtype, const float* router,
+                            const float* correction, int num_tokens, int K, int E, int top, float scale, int normalize,
+                            hipStream_t stream) {
+  if (num_tokens <= 0) return TS_OK;
+  if (K <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > MOE_MAX_TOP || top > E) return TS_BAD_SHAPE;
+  const unsigned blocks = (num_tokens + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS;
+  const size_t lds = (size_t)2 * MOE_ROUTE_TOKENS * E * sizeof(float);
+  if (x_dtype == 0)
+    moe_route_kernel<float><<<blocks, MOE_THREADS, lds, stream>>>(ids_out, w_out, (const float*)x, router, correction, num_tokens,
+                                                                  K, E, top, scale, normalize);
+  else if (x_dtype == 1)
+    moe_route_kernel<bf16_t><<<blocks, MOE_THREADS, lds, stream>>>(ids_out, w_out, (const bf16_t*)x, router, correction,
+                                                                   num_tokens, K, E, top, scale, normalize);
+  else return TS_BAD_DTYPE;
+  return ts_check_launch();
+}
+
+// One workgroup: counts per expert, their running sums, the tiles, then every pair into its expert's stretch.
+#define MOE_GROUP_THREADS 1024
+__global__ void __launch_bounds__(MOE_GROUP_THREADS)
+moe_group_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ sorted, int32_t* __restrict__ tiles, int P, int E,
+                 int tile_rows, int max_tiles) {
+  __shared__ int count_s[MOE_MAX_EXPERTS];
+  __shared__ int first_s[MOE_MAX_EXPERTS + 1];
+  __shared__ int tile_s[MOE_MAX_EXPERTS + 1];
+  for (int e = threadIdx.x; e < E; e += MOE_GROUP_THREADS) count_s[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += MOE_GROUP_THREADS) atomicAdd(&count_s[ids[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int first = 0, tile = 0;
+    for (int e = 0; e < E; ++e) {
+      first_s[e] = first;
+      tile_s[e] = tile;
+      first += count_s[e];
+      tile += (count_s[e] + tile_rows - 1) / tile_rows;
+    }
+    first_s[E] = first;
+    tile_s[E] = tile;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += MOE_GROUP_THREADS) {
+    const int n = count_s[e];
+    for (int i = 0, tile = tile_s[e]; i < n && tile < max_tiles; i += tile_rows, ++tile) {
+      tiles[3 * tile] = e;
+      tiles[3 * tile + 1] = first_s[e] + i;
+      tiles[3 * tile + 2] = min(tile_rows, n - i);
+    }
+  }
+  for (int tile = tile_s[E] + threadIdx.x; tile < max_tiles; tile += MOE_GROUP_THREADS) {
+    tiles[3 * tile] = 0;
+    tiles[3 * tile + 1] = 0;
+    tiles[3 * tile + 2] = 0;
+  }
+  // every pair into its expert's stretch, in the order the threads come by (a row's sums do not depend on its
+  // place in a tile, so the order inside an expert changes no result)
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += MOE_GROUP_THREADS) count_s[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += MOE_GROUP_THREADS) {
+    const int e = ids[p];
+    sorted[first_s[e] + atomicAdd(&count_s[e], 1)] = p;
+  }
+}
+
+extern "C" int ts_moe_group(const int32_t* ids, int32_t* sorted, int32_t* tiles, int P, int E, int tile_rows, int max_tiles,
+                            hipStream_t stream) {
+  if (P <= 0) return TS_OK;
+  // (tiles of a step: at most P / tile_rows full ones and one partly filled per expert that has pairs)
+  if (E <= 0 || E > MOE_MAX_EXPERTS || tile_rows <= 0 || max_tiles < P / tile_rows + (E < P ? E : P)) return TS_BAD_SHAPE;
+  moe_group_kernel<<<1, MOE_GROUP_THREADS, 0, stream>>>(ids, sorted, tiles, P, E, tile_rows, max_tiles);
+  return ts_check_launch();
+}
+
+#define MOE_BM 16
+#define MOE_BN 64
+#define MOE_KC 32
+
+static __device__ __forceinline__ float moe_unit(float g, float u, float limit, float slope, float shift) {
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  return g / (1.0f + expf(-slope * g)) * (u + shift);
+}
+
+// Plain 32-bit multiply-adds: a tile of up to 16 rows by 64 columns a workgroup; thread (column, row quarter).
+template <typename TX, typename TO>
+__global__ void __launch_bounds__(MOE_THREADS)
+moe_gemm_kernel(TO* __restrict__ out, const TX* __restrict__ x, const TX* __restrict__ w, const int32_t* __restrict__ sorted,
+                const int32_t* __restrict__ tiles, int src_div, int N, int K, int glu, float limit, float slope, float shift) {
+  __shared__ float x_s[MOE_BM][MOE_KC + 1];
+  __shared__ float w_s[2][MOE_BN][MOE_KC + 1];
+  __shared__ int row_s[MOE_BM];
+  const int tile = blockIdx.x;
+  const int rows = tiles[3 * tile + 2];
+  if (rows == 0) return;
+  const int e = tiles[3 * tile], first = tiles[3 * tile + 1];
+  const int n0 = blockIdx.y * MOE_BN;
+  const int tx = threadIdx.x & (MOE_BN - 1), ty = threadIdx.x / MOE_BN;
+  if (threadIdx.x < MOE_BM) row_s[threadIdx.x] = threadIdx.x < rows ? sorted[first + threadIdx.x] : -1;
+  __syncthreads();
+  const int64_t expert_rows = glu ? 2 * (int64_t)N : N;
+  const TX* we = w + (int64_t)e * expert_rows * K;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f}, acc2[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += MOE_KC) {
+    for (int i = threadIdx.x; i < MOE_BM * MOE_KC; i += MOE_THREADS) {
+      const int r = i / MOE_KC, kk = i - r * MOE_KC;
+      const int p = row_s[r];
+      x_s[r][kk] = (p >= 0 && k0 + kk < K) ? Num<TX>::ld(x + (int64_t)(p / src_div) * K + k0 + kk) : 0.f;
+    }
+    for (int i = threadIdx.x; i < MOE_BN * MOE_KC; i += MOE_THREADS) {
+      const int c = i / MOE_KC, kk = i - c * MOE_KC;
+      const bool in = n0 + c < N && k0 + kk < K;
+      w_s[0][c][kk] = in ? Num<TX>::ld(we + (int64_t)(n0 + c) * K + k0 + kk) : 0.f;
+      if (glu) w_s[1][c][kk] = in ? Num<TX>::ld(we + (int64_t)(N + n0 + c) * K + k0 + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < MOE_KC; ++kk) {
+      const float wv = w_s[0][tx][kk];
+      const float wu = glu ? w_s[1][tx][kk] : 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float xv = x_s[ty * 4 + r][kk];
+        acc[r] = fmaf(xv, wv, acc[r]);
+        acc2[r] = fmaf(xv, wu, acc2[r]);
+      }
+    }
+    __syncthreads();
+  }
+  if (n0 + tx >= N) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int p = row_s[ty * 4 + r];
+    if (p < 0) continue;
+    const float y = glu ? moe_unit(acc[r], acc2[r], limit, slope, shift) : acc[r];
+    Num<TO>::st(out + (int64_t)p * N + n0 + tx, y);
+  }
+}
+
+extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype, const void* w, const int32_t* sorted,
+                           const int32_t* tiles, int max_tiles, int src_div, int N, int K, int glu, float limit, float slope,
+                           float shift, hipStream_t stream) {
+  if (max_tiles <= 0) return TS_OK;
+  if (N <= 0 || K <= 0 || src_div <= 0) return TS_BAD_SHAPE;
+  dim3 grid(max_tiles, (N + MOE_BN - 1) / MOE_BN);
+  if (grid.y > 65535) return TS_BAD_SHAPE;
+#define MOE_LAUNCH(TX, TO) \
+  moe_gemm_kernel<TX, TO><<<grid, MOE_THREADS, 0, stream>>>((TO*)out, (const TX*)x, (const TX*)w, sorted, tiles, src_div, N, K, \
+                                                            glu, limit, slope, shift)
+  if (x_dtype == 0 && out_dtype == 0) MOE_LAUNCH(float, float);
+  else if (x_dtype == 1 && out_dtype == 1) MOE_LAUNCH(bf16_t, bf16_t);
+  else if (x_dtype == 1 && out_dtype == 0) MOE_LAUNCH(bf16_t, float);
+  else return TS_BAD_DTYPE;
+#undef MOE_LAUNCH
+  return ts_check_launch();
+}
+
+__global__ void __launch_bounds__(MOE_THREADS)
+moe_combine_kernel(float* __restrict__ out, const float* __restrict__ rows, const float* __restrict__ weights,
+                   const float* __restrict__ shared, int width, int top) {
+  const int64_t t = blockIdx.x;
+  for (int i = threadIdx.x; i < width; i += MOE_THREADS) {
+    float acc = 0.f;
+    for (int j = 0; j < top; ++j) acc = fmaf(weights[t * top + j], rows[(t * top + j) * width + i], acc);
+    if (shared) acc += shared[t * width + i];
+    out[t * width + i] = acc;
+  }
+}
+
+extern "C" int ts_moe_combine(float* out, const float* rows, const float* weights, const float* shared, int num_tokens,
+                              int width, int top, hipStream_t stream) {
+  if (num_tokens <= 0) return TS_OK;
+  if (width <= 0 || top <= 0) return TS_BAD_SHAPE;
+  moe_combine_kernel<<<num_tokens, MOE_THREADS, 0, stream>>>(out, rows, weights, shared, width, top);
+  return ts_check_launch();
+}

@@ -1,0 +1,143 @@
+// What lies between a q|k|v projection and the cache for mixers whose projected rows first pass a short causal
+// convolution over time, channel by channel:
+//   y_t[c] = sum_j w[c][j] u_(t - taps + 1 + j)[c],    j = 0 .. taps - 1,
+// with zeros before a request's first token. The last taps - 1 projected rows of every request are its state
+// ([slots, taps - 1, channels], oldest first, zero at admission): a step's first tokens reach back into it.
+//   * `ts_conv_finish`: the convolution; then, optionally, every q and k head divided by its root mean square
+//     and scaled by a weight shared by all heads; q times 1 + coef ln(floor((p + 1) / every) + 1) at position p
+//     (coef 0: not); q goes to [tokens, heads, dim], k and v to their cache slots. Key and value heads may
+//     differ in size; a mixer that reads another's cache has q channels only (nkv = 0).
+//   * `ts_conv_state_update`: after it, the state moves on by the step's rows (its own launch, so that no row
+//     of the state is overwritten while a token of the step still reads it).
+// Everything is 32-bit up to the store.
+#include "common.h"
+
+#define SC_WAVES 4
+#define SC_MAX_HD 256
+#define SC_MAX_TAPS 16
+
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(SC_WAVES * TS_WAVE)
+conv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restrict__ v_cache, const TI* __restrict__ proj,
+                   int64_t row_stride, const float* __restrict__ conv_w, const float* __restrict__ state,
+                   const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+                   const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
+                   const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots,
+                   const int32_t* __restrict__ slots, int nh, int nkv, int hd, int vd_size, int taps, float temp_coef,
+                   int temp_every, int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh,
+                   int64_t vd) {
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
+  const int t = blockIdx.x;
+  const int heads = nh + 2 * nkv;
+  const int channels = (nh + nkv) * hd + nkv * vd_size;
+  const int pos = positions[t];
+  const int seq = seq_of_token[t];
+  const int first = cu_seqlens[seq];                   // the step's first token of this request
+  const int local = t - first;                         // tokens of the step before this one
+  const float* st = taps > 1 ? state + (int64_t)state_slots[seq] * (taps - 1) * channels : nullptr;
+  const int slot = slots ? slots[t] : -1;
+  const bool stores = slot >= 0 && k_cache;
+  const int page = stores ? slot / page_size : 0, off = stores ? slot - page * page_size : 0;
+  float temp = 1.0f;
+  if (temp_coef != 0.f) temp = 1.0f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.0f);
+  for (int h = wave; h < heads; h += SC_WAVES) {
+    const bool is_q = h < nh, is_v = h >= nh + nkv;
+    if (!is_q && !stores) continue;
+    const int size = is_v ? vd_size : hd;
+    const int c0 = is_v ? (nh + nkv) * hd + (h - nh - nkv) * vd_size : h * hd;
+    float y[SC_MAX_HD / TS_WAVE];
+    float squares = 0.f;
+#pragma unroll
+    for (int i = 0; i < SC_MAX_HD / TS_WAVE; ++i) {
+      const int d = lane + i * TS_WAVE;
+      float acc = 0.f;
+      if (d < size) {
+        const int c = c0 + d;
+        for (int j = 0; j < taps; ++j) {
+          const int back = taps - 1 - j;                // rows before this token
+          float u;
+          if (back <= local) u = Num<TI>::ld(proj + (int64_t)(t - back) * row_stride + c);
+          else u = st[(int64_t)(taps - 1 - (back - local)) * channels + c];
+          acc = fmaf(conv_w[(int64_t)c * taps + j], u, acc);
+        }
+      }
+      y[i] = acc;
+      squares = fmaf(acc, acc, squares);
+    }
+    const float* nw = is_v ? nullptr : (is_q ? q_norm_w : k_norm_w);
+    float scale = 1.0f;
+    if (nw) scale = 1.0f / sqrtf(wave_sum(squares) / (float)size + eps);
+    if (is_q) scale *= temp;
+    TO* dst = is_q ? q_out + ((int64_t)t * nh + h) * hd
+              : !is_v ? k_cache + page * kp + off * ks + (int64_t)(h - nh) * kh
+                      : v_cache + page * vp + off * vs + (int64_t)(h - nh - nkv) * vh;
+    const int64_t step = is_v ? vd : 1;
+#pragma unroll
+    for (int i = 0; i < SC_MAX_HD / TS_WAVE; ++i) {
+      const int d = lane + i * TS_WAVE;
+      if (d < size) Num<TO>::st(dst + (int64_t)d * step, y[i] * scale * (nw ? nw[d] : 1.0f));
+    }
+  }
+}
+
+// A thread per (request of the step, channel): row i of the new state is the row that lies taps - 1 - i rows
+// before the end of (old state rows, the step's rows). Ascending i reads only rows not yet overwritten.
+template <typename TI>
+__global__ void __launch_bounds__(SC_WAVES * TS_WAVE)
+conv_state_update_kernel(float* __restrict__ state, const TI* __restrict__ proj, int64_t row_stride,
+                         const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, int num_seqs,
+                         int channels, int taps) {
+  const int64_t gid = (int64_t)blockIdx.x * (SC_WAVES * TS_WAVE) + threadIdx.x;
+  if (gid >= (int64_t)num_seqs * channels) return;
+  const int seq = (int)(gid / channels), c = (int)(gid - (int64_t)seq * channels);
+  const int first = cu_seqlens[seq], n = cu_seqlens[seq + 1] - first;
+  if (n <= 0) return;
+  float* st = state + (int64_t)state_slots[seq] * (taps - 1) * channels;
+  for (int i = 0; i < taps - 1; ++i) {
+    const int src = n - (taps - 1) + i;                 // index among the step's rows; below 0: still an old row
+    const float v = src >= 0 ? Num<TI>::ld(proj + (int64_t)(first + src) * row_stride + c) : st[(int64_t)(i + n) * channels + c];
+    st[(int64_t)i * channels + c] = v;
+  }
+}
+
+extern "C" int ts_conv_finish(void* q_out, void* k_cache, void* v_cache, const void* proj, int64_t row_stride,
+                              const float* conv_w, const float* state, const float* q_norm_w, const float* k_norm_w, float eps,
+                              const int32_t* positions, const int32_t* seq_of_token, const int32_t* cu_seqlens,
+                              const int32_t* state_slots, const int32_t* slots, int num_tokens, int nh, int nkv, int hd,
+                              int vd_size, int taps, float temp_coef, int temp_every, int page_size, int64_t kp, int64_t ks,
+                              int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int in_dtype, int out_dtype,
+                              hipStream_t stream) {
+  if (num_tokens <= 0) return TS_OK;
+  if (hd <= 0 || hd > SC_MAX_HD || vd_size <= 0 || vd_size > SC_MAX_HD || nh <= 0 || nkv < 0 || taps < 1 || taps > SC_MAX_TAPS ||
+      page_size <= 0 || (taps > 1 && !state) || (temp_coef != 0.f && temp_every <= 0) ||
+      row_stride < (int64_t)(nh + nkv) * hd + (int64_t)nkv * vd_size)
+    return TS_BAD_SHAPE;
+#define SC_LAUNCH(TI, TO) \
+  conv_finish_kernel<TI, TO><<<num_tokens, SC_WAVES * TS_WAVE, 0, stream>>>( \
+      (TO*)q_out, (TO*)k_cache, (TO*)v_cache, (const TI*)proj, row_stride, conv_w, state, q_norm_w, k_norm_w, eps, positions, \
+      seq_of_token, cu_seqlens, state_slots, slots, nh, nkv, hd, vd_size, taps, temp_coef, temp_every, page_size, kp, ks, kh, \
+      vp, vs, vh, vd)
+  if (in_dtype == 0 && out_dtype == 0) SC_LAUNCH(float, float);
+  else if (in_dtype == 0 && out_dtype == 1) SC_LAUNCH(float, bf16_t);
+  else if (in_dtype == 1 && out_dtype == 1) SC_LAUNCH(bf16_t, bf16_t);
+  else return TS_BAD_DTYPE;
+#undef SC_LAUNCH
+  return ts_check_launch();
+}
+
+extern "C" int ts_conv_state_update(float* state, const void* proj, int64_t row_stride, const int32_t* cu_seqlens,
+                                    const int32_t* state_slots, int num_seqs, int channels, int taps, int in_dtype,
+                                    hipStream_t stream) {
+  if (num_seqs <= 0 || taps <= 1) return TS_OK;
+  if (channels <= 0 || taps > SC_MAX_TAPS || row_stride < channels) return TS_BAD_SHAPE;
+  const int64_t threads = (int64_t)num_seqs * channels;
+  const unsigned blocks = (unsigned)((threads + SC_WAVES * TS_WAVE - 1) / (SC_WAVES * TS_WAVE));
+  if (in_dtype == 0)
+    conv_state_update_kernel<float><<<blocks, SC_WAVES * TS_WAVE, 0, stream>>>(state, (const float*)proj, row_stride, cu_seqlens,
+                                                                                state_slots, num_seqs, channels, taps);
+  else if (in_dtype == 1)
+    conv_state_update_kernel<bf16_t><<<blocks, SC_WAVES * TS_WAVE, 0, stream>>>(state, (const bf16_t*)proj, row_stride, cu_seqlens,
+                                                                                 state_slots, num_seqs, channels, taps);
+  else return TS_BAD_DTYPE;
+  return ts_check_launch();
+}

@@ -57,6 +57,8 @@ class Destination:
     def view(self, param):
         """The part of `param` (a tensor) that the checkpoint tensor fills, as a view."""
         t = param[self.index] if self.index else param
+        if t.dim() == 0:
+            return t                     # (one number: nothing to slice)
         t = t.narrow(0, self.row, self.rows if self.rows is not None else t.shape[0] - self.row)
         if t.dim() > 1:
             t = t.narrow(1, self.col, self.cols if self.cols is not None else t.shape[1] - self.col)

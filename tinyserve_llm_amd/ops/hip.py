@@ -85,7 +85,18 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_mingru_scan_chunks": [p, i, p, i, p, i, p, p, p, p, p, i, i, i, p],
         "ts_qkv_finish": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, f, i, f, i, i64, i64, i64, i64, i64, i64, i64, i, i, p],
         "ts_paged_attention_general": [p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, f, i, i,
-                                       i, i, p],
+                                       i, i, p, p, p, i64, p],
+        "ts_dyt": [p, i, p, i, p, i, p, i, p, p, p, p, i, i, p],
+        "ts_dyt_stream": [p, p, i, p, p, p, p, i, p, p, p, i, i, p],
+        "ts_embedding_dyt_stream": [p, p, i, p, f, p, p, p, i, i, p],
+        "ts_capped_glu": [p, i, p, i, i64, i, i, f, f, f, p],
+        "ts_conv_finish": [p, p, p, p, i64, p, p, p, p, f, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i64, i64, i64, i64, i64,
+                           i64, i64, i, i, p],
+        "ts_conv_state_update": [p, p, i64, p, p, i, i, i, i, p],
+        "ts_moe_route": [p, p, p, i, p, p, i, i, i, i, f, i, p],
+        "ts_moe_group": [p, p, p, i, i, i, i, p],
+        "ts_moe_gemm": [p, i, p, i, p, p, p, i, i, i, i, i, f, f, f, p],
+        "ts_moe_combine": [p, p, p, p, i, i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
                                      i64, i64, i64, i64, p, i, p],
     }
@@ -1749,4 +1760,270 @@ def paged_attention_general(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
         T, nh, nkv, hd, vd, k_cache.shape[1], *k_cache.stride()[:3], *v_cache.stride(), block_tables.shape[1],
         float(scale), float(softcap), int(sink), int(window), _code(q.dtype), _page_run(pages_per_entry), _stream()))
+    return out
+
+
+def paged_attention_sloped(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int, scale: float, *,
+                           window: int = 0, sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None,
+                           gate: torch.Tensor | None = None) -> torch.Tensor:
+    """Attention of a packed step over the cache in 32-bit, with what `paged_attention` has no argument for:
+    `slopes` (float32 [heads]): slopes[h] * (query position - key position) is taken off every score;
+    `sinks` (float32 [heads]): the softmax's denominator also holds exp(sinks[h]) (a key without a value);
+    `gate` (float32 [tokens, >= heads * value_dim], a view whose rows may lie apart): the output row is
+    multiplied by sigmoid(gate) element by element. out [tokens, heads, value_dim] in q's type."""
+    _gpu(q, k_cache, v_cache, sinks, slopes, gate)
+    _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
+    T, nh, hd = q.shape
+    nkv, vd = k_cache.shape[2], v_cache.shape[3]
+    _check_cache_pair(k_cache, v_cache, q.dtype, nkv, hd, vd)
+    _need(nh % nkv == 0, lambda: f"{nh} heads do not divide into {nkv} key/value heads")
+    tables, seq_of_token, positions = ctx.block_tables[space], ctx.seq_of_token, ctx.positions
+    table_page = getattr(ctx, "page_size", 0) or k_cache.shape[1]
+    _need(table_page % k_cache.shape[1] == 0, lambda: f"block tables in pages of {table_page} over a cache in pages of {k_cache.shape[1]}")
+    _need(tables.dtype == torch.int32 and tables.dim() == 2 and tables.is_contiguous(),
+          "block_tables must be contiguous int32 [requests, pages]")
+    for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
+        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), lambda: f"{name} must be int32 [tokens]")
+    for name, t in (("sinks", sinks), ("slopes", slopes)):
+        _need(t is None or (t.dtype == torch.float32 and t.shape == (nh,) and t.is_contiguous()), lambda: f"{name} must be float32 [heads]")
+    gate_stride = 0
+    if gate is not None:
+        _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape == (T, nh * vd) and gate.stride(1) == 1
+              and gate.stride(0) >= nh * vd, "the gate must be float32 [tokens, heads * value_dim] with contiguous rows")
+        gate_stride = gate.stride(0)
+    out = torch.empty((T, nh, vd), dtype=q.dtype, device=q.device)
+    _run("paged_attention_general", library().ts_paged_attention_general(
+        _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(tables), _ptr(seq_of_token), _ptr(positions),
+        T, nh, nkv, hd, vd, k_cache.shape[1], *k_cache.stride()[:3], *v_cache.stride(), tables.shape[1],
+        float(scale), 0.0, 0, int(window), _code(q.dtype), _page_run(table_page // k_cache.shape[1]), _ptr(sinks), _ptr(slopes),
+        _ptr(gate), gate_stride, _stream()))
+    return out
+
+
+# ---- the dynamic-tanh norm ----
+
+def _dyt_params(alpha: torch.Tensor, w: torch.Tensor, b: torch.Tensor, width: int) -> None:
+    _need(alpha.dtype == torch.float32 and alpha.numel() == 1, "alpha must be one float32")
+    for t in (w, b):
+        _need(t.dtype == torch.float32 and t.shape == (width,) and t.is_contiguous(), "the norm's weight and bias must be float32 [width]")
+
+
+def dyt(x: torch.Tensor, alpha: torch.Tensor, w: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype,
+        residual: torch.Tensor | None = None, rows: torch.Tensor | None = None,
+        keep_sum: bool = False) -> "tuple[torch.Tensor, torch.Tensor | None]":
+    """tanh(alpha (x + residual)) * w + b row by row, in 32-bit, stored as `out_dtype`; with `rows`
+    (int32) only those rows, in that order; with `keep_sum` x + residual comes back as well, in x's type."""
+    _gpu(x, alpha, w, b, residual, rows)
+    _need(x.dim() == 2 and x.is_contiguous(), "the input must be contiguous [tokens, width]")
+    _dyt_params(alpha, w, b, x.shape[1])
+    _need(residual is None or (residual.shape == x.shape and residual.is_contiguous()), "the residual must match the input")
+    _need(rows is None or residual is None, "picked rows are normalised, not summed")
+    n = x.shape[0]
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.dim() == 1 and rows.is_contiguous(), "rows must be int32")
+        n = rows.shape[0]
+    out = torch.empty((n, x.shape[1]), dtype=out_dtype, device=x.device)
+    total = torch.empty_like(x) if keep_sum and residual is not None else None
+    _run("dyt", library().ts_dyt(_ptr(out), _code(out_dtype), _ptr(x), _code(x.dtype), _ptr(residual),
+                                 0 if residual is None else _code(residual.dtype), _ptr(total), _code(x.dtype), _ptr(alpha),
+                                 _ptr(w), _ptr(b), _ptr(rows), n, x.shape[1], _stream()))
+    return out, total
+
+
+def dyt_stream(x: torch.Tensor, a: torch.Tensor | None, post: "tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None",
+               pre: "tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None", out_dtype: torch.dtype) -> torch.Tensor | None:
+    """The float32 stream x [tokens, width] takes x += n_post(a) in place (`a`: what a branch made, float32
+    or bfloat16; n_post(a) = tanh(alpha a) w + b with `post` = (alpha, w, b), or a itself if `post` is None),
+    and n_pre(x) of the updated rows comes back in `out_dtype` if `pre` is given."""
+    _gpu(x, a)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "the stream must be contiguous float32 [tokens, width]")
+    _need(a is None or (a.shape == x.shape and a.is_contiguous()), "the branch's rows must match the stream")
+    _need(post is None or a is not None, "a norm after a branch needs the branch's rows")
+    for params in (post, pre):
+        if params is not None:
+            _gpu(*params)
+            _dyt_params(*params, x.shape[1])
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device) if pre is not None else None
+    nothing = (None, None, None)
+    _run("dyt_stream", library().ts_dyt_stream(
+        _ptr(x), _ptr(a), 0 if a is None else _code(a.dtype), *(_ptr(t) for t in (post or nothing)), _ptr(out), _code(out_dtype),
+        *(_ptr(t) for t in (pre or nothing)), x.shape[0], x.shape[1], _stream()))
+    return out
+
+
+def embedding_dyt_stream(table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0,
+                         norm: "tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None" = None) -> torch.Tensor:
+    """out[t] = n(table[ids[t]] * scale) as float32 rows (n: a dynamic-tanh norm (alpha, w, b), or none):
+    the start of a residual stream that is kept in 32-bit."""
+    _gpu(table, ids)
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [vocab, hidden]")
+    _need(ids.dtype == torch.int32 and ids.dim() == 1 and ids.is_contiguous(), "ids must be int32 [tokens]")
+    if norm is not None:
+        _gpu(*norm)
+        _dyt_params(*norm, table.shape[1])
+    out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32, device=table.device)
+    _run("embedding_dyt_stream", library().ts_embedding_dyt_stream(
+        _ptr(out), _ptr(table), _code(table.dtype), _ptr(ids), float(scale), *(_ptr(t) for t in (norm or (None, None, None))),
+        ids.shape[0], table.shape[1], _stream()))
+    return out
+
+
+def capped_glu(gate_up: torch.Tensor, limit: float, slope: float, up_shift: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """From rows [gate | up] (float32 or `out_dtype`): g = min(gate, limit), u = clamp(up, -limit, limit)
+    (limit <= 0: no cap), y = g sigmoid(slope g) (u + up_shift), in 32-bit, stored as `out_dtype`."""
+    _gpu(gate_up)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0 and gate_up.stride(1) == 1 and gate_up.stride(0) >= gate_up.shape[1],
+          "the input must be [tokens, 2 ff] with contiguous rows")
+    n, ff = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((n, ff), dtype=out_dtype, device=gate_up.device)
+    _run("capped_glu", library().ts_capped_glu(_ptr(out), _code(out_dtype), _ptr(gate_up), _code(gate_up.dtype), gate_up.stride(0),
+                                               n, ff, float(limit), float(slope), float(up_shift), _stream()))
+    return out
+
+
+# ---- a short convolution between projection and cache ----
+
+CONV_MAX_TAPS = 16
+
+
+def conv_finish(proj: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor | None, ctx, slots: torch.Tensor | None,
+                k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, num_heads: int, num_kv_heads: int, head_dim: int,
+                value_dim: int, out_dtype: torch.dtype, *, q_norm: torch.Tensor | None = None, k_norm: torch.Tensor | None = None,
+                eps: float = 0.0, temp_coef: float = 0.0, temp_every: int = 1) -> torch.Tensor:
+    """From projected rows (float32 or `out_dtype`, [tokens, >= channels], the channels q | k | v leading each
+    row; `num_kv_heads` 0: q only) to q [tokens, heads, head_dim] and the cache slots of k and v: every channel
+    first passes the causal convolution y_t = sum_j conv_w[c, j] u_(t - taps + 1 + j) over its request's rows,
+    those before the step taken from `state` ([slots, taps - 1, channels] float32, oldest first); then q and k
+    heads are divided by their root mean square and scaled by `q_norm` / `k_norm` ([head_dim] float32; None:
+    not), and q is multiplied by 1 + temp_coef ln(floor((p + 1) / temp_every) + 1). The state is moved on by
+    `conv_state_update`, which the caller runs after this."""
+    _gpu(proj, conv_w, state, slots, k_cache, v_cache, q_norm, k_norm)
+    T = proj.shape[0]
+    channels = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
+    _need(proj.dim() == 2 and proj.shape[1] >= channels and proj.stride(1) == 1 and proj.stride(0) >= proj.shape[1],
+          lambda: f"the projected rows must be [tokens, >= {channels}] with contiguous rows")
+    _need(proj.dtype in (torch.float32, out_dtype), "the projected rows are float32 or of the output's type")
+    _need(conv_w.dtype == torch.float32 and conv_w.dim() == 2 and conv_w.shape[0] == channels and conv_w.is_contiguous()
+          and 1 <= conv_w.shape[1] <= CONV_MAX_TAPS, lambda: f"the convolution's weights must be float32 [{channels}, taps <= {CONV_MAX_TAPS}]")
+    taps = conv_w.shape[1]
+    if taps > 1:
+        _need(state is not None and state.dtype == torch.float32 and state.dim() == 3 and state.shape[1:] == (taps - 1, channels)
+              and state.is_contiguous(), lambda: f"the state must be float32 [slots, {taps - 1}, {channels}]")
+    _need(0 < head_dim <= 256 and 0 < value_dim <= 256, "head sizes up to 256")
+    for name, t, n in (("positions", ctx.positions, T), ("seq_of_token", ctx.seq_of_token, T), ("cu_seqlens", ctx.cu_seqlens, ctx.num_seqs + 1),
+                       ("state_slots", ctx.state_slots, ctx.num_seqs)):
+        _need(t.dtype == torch.int32 and t.shape == (n,) and t.is_contiguous(), lambda: f"{name} must be int32 [{n}]")
+    for name, t in (("q_norm", q_norm), ("k_norm", k_norm)):
+        _need(t is None or (t.dtype == torch.float32 and t.shape == (head_dim,) and t.is_contiguous()), lambda: f"{name} must be float32 [head_dim]")
+    _need(temp_coef == 0.0 or temp_every >= 1, "the query multiplier's period is at least 1")
+    page_size, kst, vst = 1, (0, 0, 0), (0, 0, 0, 0)
+    if k_cache is not None:
+        _need(num_kv_heads > 0 and v_cache is not None and slots is not None, "a cache write needs k, v and the slots")
+        _need(slots.dtype == torch.int32 and slots.shape == (T,) and slots.is_contiguous(), "slots must be int32 [tokens]")
+        _check_cache_pair(k_cache, v_cache, out_dtype, num_kv_heads, head_dim, value_dim)
+        page_size, kst, vst = k_cache.shape[1], k_cache.stride()[:3], v_cache.stride()
+    else:
+        _need(num_kv_heads == 0, "key and value channels need a cache to go to")
+    q = torch.empty((T, num_heads, head_dim), dtype=out_dtype, device=proj.device)
+    _run("conv_finish", library().ts_conv_finish(
+        _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(proj), proj.stride(0), _ptr(conv_w), _ptr(state), _ptr(q_norm), _ptr(k_norm),
+        float(eps), _ptr(ctx.positions), _ptr(ctx.seq_of_token), _ptr(ctx.cu_seqlens), _ptr(ctx.state_slots), _ptr(slots), T,
+        num_heads, num_kv_heads, head_dim, value_dim, taps, float(temp_coef), int(temp_every), page_size, *kst, *vst,
+        _code(proj.dtype), _code(out_dtype), _stream()))
+    return q
+
+
+def conv_state_update(state: torch.Tensor, proj: torch.Tensor, ctx) -> None:
+    """Moves every request's convolution state ([slots, taps - 1, channels] float32) on by the step's
+    projected rows: afterwards it holds the last taps - 1 rows of (what it held, the step's rows)."""
+    _gpu(state, proj)
+    _need(state.dtype == torch.float32 and state.dim() == 3 and state.is_contiguous(), "the state must be contiguous float32 [slots, taps - 1, channels]")
+    channels, taps = state.shape[2], state.shape[1] + 1
+    _need(proj.dim() == 2 and proj.shape[1] >= channels and proj.stride(1) == 1 and proj.stride(0) >= proj.shape[1],
+          "the projected rows must have contiguous rows that lead with the channels")
+    _need(taps <= CONV_MAX_TAPS, lambda: f"up to {CONV_MAX_TAPS} taps")
+    _run("conv_state_update", library().ts_conv_state_update(
+        _ptr(state), _ptr(proj), proj.stride(0), _ptr(ctx.cu_seqlens), _ptr(ctx.state_slots), ctx.num_seqs, channels, taps,
+        _code(proj.dtype), _stream()))
+
+
+# ---- a mixture of experts ----
+
+MOE_TILE_ROWS = 16
+MOE_MAX_EXPERTS = 1024
+MOE_MAX_TOP = 32
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor | None, top: int, scale: float,
+              normalize: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
+    """(experts int32 [tokens, top], weights float32 [tokens, top]): scores s = sigmoid(x · routerᵀ) in 32-bit;
+    the `top` experts with the largest s + correction; weights s of the chosen, over their sum (+ 1e-20) if
+    `normalize`, times `scale`."""
+    _gpu(x, router, correction)
+    _need(x.dim() == 2 and x.is_contiguous(), "the input must be contiguous [tokens, width]")
+    E = router.shape[0]
+    _need(router.dtype == torch.float32 and router.shape == (E, x.shape[1]) and router.is_contiguous(), "the router must be float32 [experts, width]")
+    _need(correction is None or (correction.dtype == torch.float32 and correction.shape == (E,) and correction.is_contiguous()),
+          "the correction must be float32 [experts]")
+    _need(1 <= top <= min(E, MOE_MAX_TOP) and E <= MOE_MAX_EXPERTS, lambda: f"1 <= top <= min(experts, {MOE_MAX_TOP}), experts <= {MOE_MAX_EXPERTS}")
+    ids = torch.empty((x.shape[0], top), dtype=torch.int32, device=x.device)
+    weights = torch.empty((x.shape[0], top), dtype=torch.float32, device=x.device)
+    _run("moe_route", library().ts_moe_route(_ptr(ids), _ptr(weights), _ptr(x), _code(x.dtype), _ptr(router), _ptr(correction),
+                                             x.shape[0], x.shape[1], E, top, float(scale), int(normalize), _stream()))
+    return ids, weights
+
+
+class ExpertTiles:
+    """A step's (token, choice) pairs grouped by expert: `sorted` int32 [pairs] (pair indices, an expert's
+    side by side), `tiles` int32 [max_tiles, 3] = (expert, first index into `sorted`, rows; rows 0: unused)."""
+
+    def __init__(self, sorted_pairs: torch.Tensor, tiles: torch.Tensor, top: int, experts: int) -> None:
+        self.sorted, self.tiles, self.top, self.experts = sorted_pairs, tiles, top, experts
+
+
+def moe_group(ids: torch.Tensor, experts: int) -> ExpertTiles:
+    _gpu(ids)
+    _need(ids.dtype == torch.int32 and ids.dim() == 2 and ids.is_contiguous(), "the chosen experts must be contiguous int32 [tokens, top]")
+    _need(0 < experts <= MOE_MAX_EXPERTS, lambda: f"up to {MOE_MAX_EXPERTS} experts")
+    P = ids.numel()
+    max_tiles = P // MOE_TILE_ROWS + min(experts, P)
+    sorted_pairs = torch.empty((P,), dtype=torch.int32, device=ids.device)
+    tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=ids.device)
+    _run("moe_group", library().ts_moe_group(_ptr(ids), _ptr(sorted_pairs), _ptr(tiles), P, experts, MOE_TILE_ROWS, max_tiles, _stream()))
+    return ExpertTiles(sorted_pairs, tiles, ids.shape[1], experts)
+
+
+def moe_gemm(x: torch.Tensor, weights: torch.Tensor, grouped: ExpertTiles, out_dtype: torch.dtype, *, per_token: bool,
+             glu: "tuple[float, float, float] | None" = None) -> torch.Tensor:
+    """out[pair] = x[row of the pair] · weights[expert of the pair]ᵀ for every pair of the step; `per_token`:
+    x holds a row per token (a pair reads its token's), else a row per pair. weights [experts, n, k]; with
+    `glu` = (limit, slope, up_shift) they hold gate rows then up rows (n = 2 ff) and the capped gated unit of
+    the two sums leaves: out [pairs, ff]."""
+    _gpu(x, weights)
+    P = grouped.sorted.shape[0]
+    _need(x.dim() == 2 and x.is_contiguous() and x.shape[0] == (P // grouped.top if per_token else P), "the operand must be contiguous, a row per token or per pair")
+    _need(weights.dim() == 3 and weights.is_contiguous() and weights.shape[0] == grouped.experts and weights.shape[2] == x.shape[1]
+          and weights.dtype == x.dtype, "the experts' matrices must be contiguous [experts, n, k] of the operand's type")
+    n = weights.shape[1]
+    if glu is not None:
+        _need(n % 2 == 0, "gate rows and up rows: an even number")
+        n //= 2
+    out = torch.empty((P, n), dtype=out_dtype, device=x.device)
+    limit, slope, shift = glu if glu is not None else (0.0, 0.0, 0.0)
+    _run("moe_gemm", library().ts_moe_gemm(_ptr(out), _code(out_dtype), _ptr(x), _code(x.dtype), _ptr(weights), _ptr(grouped.sorted),
+                                           _ptr(grouped.tiles), grouped.tiles.shape[0], grouped.top if per_token else 1, n, x.shape[1],
+                                           int(glu is not None), float(limit), float(slope), float(shift), _stream()))
+    return out
+
+
+def moe_combine(rows: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = sum_j weights[t, j] * rows[t * top + j] (+ shared[t]), float32."""
+    _gpu(rows, weights, shared)
+    T, top = weights.shape
+    _need(rows.dtype == torch.float32 and rows.dim() == 2 and rows.shape[0] == T * top and rows.is_contiguous(), "rows must be contiguous float32 [tokens * top, width]")
+    _need(weights.dtype == torch.float32 and weights.is_contiguous(), "weights must be contiguous float32 [tokens, top]")
+    _need(shared is None or (shared.dtype == torch.float32 and shared.shape == (T, rows.shape[1]) and shared.is_contiguous()),
+          "the shared rows must be contiguous float32 [tokens, width]")
+    out = torch.empty((T, rows.shape[1]), dtype=torch.float32, device=rows.device)
+    _run("moe_combine", library().ts_moe_combine(_ptr(out), _ptr(rows), _ptr(weights), _ptr(shared), T, rows.shape[1], top, _stream()))
     return out

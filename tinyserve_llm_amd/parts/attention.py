@@ -14,7 +14,7 @@ from __future__ import annotations
 import torch
 
 from tinyserve_llm_amd.ops import hip
-from tinyserve_llm_amd.parts.base import KVSpec, LayerMemory, Mixer, ParamSpec, StepContext, register
+from tinyserve_llm_amd.parts.base import KVSpec, LayerMemory, Mixer, ParamSpec, StateSpec, StepContext, register
 from tinyserve_llm_amd.parts.linear import DeferredNorm, linear, streaming_copy
 
 
@@ -193,3 +193,105 @@ class GeneralAttention(Mixer):
                                 sink=self.sink)
         return linear(o.view(ctx.num_tokens, self.num_heads * self.value_dim), self.o, out_dtype=torch.float32,
                       packed=self.o_packed)
+
+
+@register("mixer", "attention_conv")
+class ConvAttention(Mixer):
+    """Grouped-query attention without rotation whose projected q, k and v rows first pass a short causal
+    convolution over time (`conv_taps` taps per channel; the last taps - 1 projected rows of a request are
+    its state), every option a constructor argument: q and k heads divided by their root mean square and
+    scaled by a weight shared by all heads (`qk_norm_eps`), q multiplied by
+    1 + q_temp_coef ln(floor((p + 1) / q_temp_every) + 1) at position p, a penalty on distance
+    2^(-slope_exponent (h + 1) / heads) * (i - j) taken off head h's scores (`slope_exponent` None: not), a
+    window, a learned per-head sink in the softmax's denominator (`sink`), and the heads' output multiplied
+    by sigmoid(W_g x) before the output projection (`gate`). `own_kv` False: the mixer projects queries (and
+    the gate) only and reads the cache of another run of the order. `cache_window`: how long the cache keeps
+    keys where other runs read it through wider windows than this one's (None: `window`). One fused
+    projection gives q | k | v | gate, 32-bit on its way out; convolution, norms, scores, weights and the
+    gate are 32-bit in every storage type."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int | None = None,
+                 conv_taps: int = 1, own_kv: bool = True, scale: float | None = None, window: int = 0,
+                 cache_window: int | None = None, qk_norm_eps: float | None = None, q_temp_coef: float = 0.0,
+                 q_temp_every: int = 1, slope_exponent: float | None = None, sink: bool = False, gate: bool = False) -> None:
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads do not divide into {num_kv_heads} key/value heads")
+        value_dim = head_dim if value_dim is None else value_dim
+        if not (0 < head_dim <= 256 and 0 < value_dim <= 256):
+            raise ValueError(f"head sizes {head_dim} / {value_dim}: the attention kernels take up to 256")
+        if not 1 <= conv_taps <= hip.CONV_MAX_TAPS:
+            raise ValueError(f"conv_taps {conv_taps}: 1 to {hip.CONV_MAX_TAPS}")
+        if window < 0 or q_temp_every < 1:
+            raise ValueError("window >= 0 (0: none), q_temp_every >= 1")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.value_dim, self.conv_taps, self.own_kv = head_dim, value_dim, conv_taps, own_kv
+        self.scale = scale if scale is not None else head_dim ** -0.5
+        self.window = window
+        self.cache_window = window if cache_window is None else cache_window
+        self.qk_norm_eps, self.q_temp_coef, self.q_temp_every = qk_norm_eps, q_temp_coef, q_temp_every
+        self.slope_exponent, self.has_sink, self.has_gate = slope_exponent, sink, gate
+        self.proj: torch.Tensor | None = None
+        self.o: torch.Tensor | None = None
+        self.conv: torch.Tensor | None = None
+        self.q_norm: torch.Tensor | None = None
+        self.k_norm: torch.Tensor | None = None
+        self.sink: torch.Tensor | None = None
+        self.slopes: torch.Tensor | None = None
+        self.proj_packed: hip.StreamingCopies | None = None
+        self.o_packed: hip.StreamingCopies | None = None
+
+    @property
+    def channels(self) -> int:
+        """Columns of the projection that pass the convolution: q, and k and v where the mixer makes its own."""
+        own = self.num_kv_heads * (self.head_dim + self.value_dim) if self.own_kv else 0
+        return self.num_heads * self.head_dim + own
+
+    @property
+    def out_size(self) -> int:
+        return self.num_heads * self.value_dim
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        specs = {"proj": ParamSpec((self.channels + (self.out_size if self.has_gate else 0), self.hidden_size)),
+                 "o": ParamSpec((self.hidden_size, self.out_size)),
+                 "conv": ParamSpec((self.channels, self.conv_taps), "float32", init=(1.0 / self.conv_taps, 0.3))}
+        if self.qk_norm_eps is not None:
+            specs["q_norm"] = ParamSpec((self.head_dim,), "float32", init=(1.0, 0.1))
+            if self.own_kv:
+                specs["k_norm"] = ParamSpec((self.head_dim,), "float32", init=(1.0, 0.1))
+        if self.has_sink:
+            specs["sink"] = ParamSpec((self.num_heads,), "float32", init=(0.0, 1.0))
+        return specs
+
+    def bind(self, params) -> None:
+        super().bind(params)
+        if self.slope_exponent is not None:
+            slopes = [2.0 ** (-self.slope_exponent * (h + 1) / self.num_heads) for h in range(self.num_heads)]
+            self.slopes = torch.tensor(slopes, dtype=torch.float32).to(self.proj.device)
+
+    def kv_spec(self) -> KVSpec:
+        return KVSpec(self.num_kv_heads, self.head_dim, self.cache_window,
+                      None if self.value_dim == self.head_dim else self.value_dim)
+
+    def state_spec(self) -> StateSpec | None:
+        return StateSpec((self.conv_taps - 1, self.channels), torch.float32) if self.conv_taps > 1 else None
+
+    def keep_streaming_copies(self) -> int:
+        self.proj_packed, self.o_packed = streaming_copy(self.proj), streaming_copy(self.o)
+        return sum(c.nbytes() for c in (self.proj_packed, self.o_packed) if c is not None)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
+        if self.own_kv != mem.store:
+            raise ValueError("a mixer with keys and values of its own writes its cache; one without reads another's")
+        proj = linear(x, self.proj, out_dtype=torch.float32, packed=self.proj_packed)
+        store = (ctx.slot_mapping[mem.space], mem.k_cache, mem.v_cache) if self.own_kv else (None, None, None)
+        q = hip.conv_finish(proj, self.conv, mem.state, ctx, *store, self.num_heads, self.num_kv_heads if self.own_kv else 0,
+                            self.head_dim, self.value_dim, x.dtype, q_norm=self.q_norm, k_norm=self.k_norm,
+                            eps=self.qk_norm_eps or 0.0, temp_coef=self.q_temp_coef, temp_every=self.q_temp_every)
+        if self.conv_taps > 1:
+            hip.conv_state_update(mem.state, proj, ctx)
+        o = hip.paged_attention_sloped(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, window=self.window,
+                                       sinks=self.sink, slopes=self.slopes,
+                                       gate=proj[:, self.channels:] if self.has_gate else None)
+        return linear(o.view(ctx.num_tokens, self.out_size), self.o, out_dtype=torch.float32, packed=self.o_packed)

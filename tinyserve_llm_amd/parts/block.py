@@ -132,3 +132,25 @@ def parallel_block(layer: Layer, hidden, residual, ctx: StepContext, mem: LayerM
     else:
         b, bias = ff.forward(h2, ctx), None
     return ResidualStream(x, a, b, bias, float(layer.block_args.get("residual_mult", 1.0))), None
+
+
+@register("block", "sandwich")
+@uses_norms("norm1", "norm1b")
+@keeps_stream
+def sandwich_block(layer: Layer, hidden, residual, ctx: StepContext, mem: LayerMemory):
+    """x <- x + norm1b(mixer(norm1(x))), then x <- x + norm2b(feed_forward(norm2(x))): a norm before and
+    one after every part ("norm2", "norm2b" only where the layer has a feed-forward). The stream is
+    32-bit; each sum is left pending in it, with the norm that the branch's rows still have to pass, so
+    that whoever takes the stream next does both norms and the sum in one kernel."""
+    from tinyserve_llm_amd.parts.stream import ResidualStream
+    if not isinstance(hidden, ResidualStream) or residual is not None:
+        raise TypeError("the sandwich arrangement runs on a 32-bit residual stream (ModelSpec.residual_dtype = 'float32')")
+    norms = layer.norms
+    x, h = hidden.take(norms["norm1"], out_dtype=norms["norm1"].weight.dtype)
+    stream = ResidualStream(x, layer.mixer.forward(h, ctx, mem), post=norms["norm1b"])
+    if "norm2" not in norms:
+        if layer.feed_forward.forward(None, ctx) is not None:
+            raise KeyError("a sandwich layer with a feed-forward names the norms 'norm2' and 'norm2b'")
+        return stream, None
+    x, h = stream.take(norms["norm2"], out_dtype=norms["norm2"].weight.dtype)
+    return ResidualStream(x, layer.feed_forward.forward(h, ctx), post=norms["norm2b"]), None

@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from tinyserve_llm_amd.ops import hip
-from tinyserve_llm_amd.parts.base import Embedding, Head, ParamSpec, StepContext, register
+from tinyserve_llm_amd.parts.base import Embedding, Head, ParamSpec, PartSpec, StepContext, make, register
 from tinyserve_llm_amd.parts.linear import linear, streaming_copy
 from tinyserve_llm_amd.parts.stream import ResidualStream
 
@@ -19,20 +19,38 @@ class TableEmbedding(Embedding):
     graph_safe = True
 
     def __init__(self, vocab_size: int, hidden_size: int, init: tuple[float, float] = (0.0, 0.02),
-                 float32_stream: bool = False) -> None:
+                 float32_stream: bool = False, scale: float = 1.0, norm: "PartSpec | None" = None) -> None:
         """`float32_stream`: the rows start a residual stream that is kept in 32-bit floats
-        (`parts.stream.ResidualStream`) whatever the table's storage type."""
+        (`parts.stream.ResidualStream`) whatever the table's storage type; such rows may be multiplied
+        by `scale` and passed through a norm that works element by element (`norm`: its PartSpec; its
+        parameters are the table's, named `norm_<name>`)."""
         self.vocab_size, self.hidden_size, self.init = vocab_size, hidden_size, tuple(init)
-        self.float32_stream = float32_stream
+        self.float32_stream, self.scale = float32_stream, scale
+        if (scale != 1.0 or norm is not None) and not float32_stream:
+            raise ValueError("a scaled or normalised embedding starts a 32-bit stream (float32_stream=True)")
+        self.norm = make("norm", norm) if norm is not None else None
+        if self.norm is not None and not hasattr(self.norm, "elementwise"):
+            raise ValueError(f"the embedding takes a norm that works element by element, not {norm.kind!r}")
         self.weight: torch.Tensor | None = None
 
     def param_specs(self) -> dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.vocab_size, self.hidden_size), init=self.init)}
+        specs = {"weight": ParamSpec((self.vocab_size, self.hidden_size), init=self.init)}
+        if self.norm is not None:
+            specs.update({f"norm_{name}": ps for name, ps in self.norm.param_specs().items()})
+        return specs
+
+    def bind(self, params) -> None:
+        super().bind({n: t for n, t in params.items() if not n.startswith("norm_")})
+        if self.norm is not None:
+            self.norm.bind({n[len("norm_"):]: t for n, t in params.items() if n.startswith("norm_")})
 
     def table(self) -> torch.Tensor | None:
         return self.weight
 
     def forward(self, ctx: StepContext) -> "torch.Tensor | ResidualStream":
+        if self.float32_stream and (self.scale != 1.0 or self.norm is not None):
+            return ResidualStream(hip.embedding_dyt_stream(self.weight, ctx.token_ids, self.scale,
+                                                           self.norm.elementwise() if self.norm is not None else None))
         if self.float32_stream:
             return ResidualStream(hip.embedding_stream(self.weight, ctx.token_ids))
         return hip.embedding(self.weight, ctx.token_ids)      # (ids are checked against the vocabulary on the host)

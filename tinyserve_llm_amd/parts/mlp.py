@@ -86,6 +86,38 @@ class DenseMLP(FeedForward):
         return down if self.down_bias is None else hip.bias_activation(down, self.down_bias, "none", torch.float32)
 
 
+@register("feed_forward", "capped_glu")
+class CappedGLU(FeedForward):
+    """A gated feed-forward with capped branches: g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
+    W_down (g sigmoid(slope g) (u + up_shift)); limit <= 0: no cap. One fused projection gives gate | up as
+    32-bit sums; the unit is taken in 32-bit and rounded to the storage type for the down projection, whose
+    result is 32-bit."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float = 0.0, slope: float = 1.702,
+                 up_shift: float = 1.0) -> None:
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.limit, self.slope, self.up_shift = limit, slope, up_shift
+        self.gate_up: torch.Tensor | None = None
+        self.down: torch.Tensor | None = None
+        self.gate_up_packed = None
+        self.down_packed = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {"gate_up": ParamSpec((2 * self.intermediate_size, self.hidden_size)),
+                "down": ParamSpec((self.hidden_size, self.intermediate_size))}
+
+    def keep_streaming_copies(self) -> int:
+        self.gate_up_packed, self.down_packed = streaming_copy(self.gate_up), streaming_copy(self.down)
+        return sum(c.nbytes() for c in (self.gate_up_packed, self.down_packed) if c is not None)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        sums = linear(x, self.gate_up, out_dtype=torch.float32, packed=self.gate_up_packed)
+        unit = hip.capped_glu(sums, self.limit, self.slope, self.up_shift, x.dtype)
+        return linear(unit, self.down, out_dtype=torch.float32, packed=self.down_packed)
+
+
 @register("feed_forward", "none")
 class NoFeedForward(FeedForward):
     """A layer without a feed-forward: `forward` gives None, which a block's residual sum leaves out."""

@@ -1,0 +1,71 @@
+"""A mixture of experts as a feed-forward: a router scores the experts for every token, the token goes
+through the `top` best of them, and their outputs are added with the router's weights; a shared expert
+may run for every token beside them. Routing lives inside the part: a step's (token, expert) pairs are
+grouped by expert on the device (`hip.moe_group`), so that the experts' products run as one launch over
+tiles of rows and nothing comes back to the host (the part can be recorded into a graph)."""
+
+from __future__ import annotations
+
+import torch
+
+from tinyserve_llm_amd.ops import hip
+from tinyserve_llm_amd.parts.base import FeedForward, ParamSpec, StepContext, register
+from tinyserve_llm_amd.parts.mlp import CappedGLU
+
+
+@register("feed_forward", "routed_experts")
+class RoutedExperts(FeedForward):
+    """Experts of the capped gated form (`parts.mlp.CappedGLU`: limit, slope, up_shift), without biases.
+    Scores s = sigmoid(W_r h), the logits in 32-bit; the `top` experts with the largest s + correction are
+    chosen (`correction` False: largest s); their weights are their s without the correction, over the chosen
+    ones' sum (+ 1e-20) if `normalize`, times `router_scale`. `shared`: the constructor arguments of a
+    `CappedGLU` that runs for every token and is added (None: no shared expert). The experts' matrices are
+    stacked: gate_up [experts, 2 ff, hidden], down [experts, hidden, ff]."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_experts: int, top: int, intermediate_size: int, limit: float = 0.0,
+                 slope: float = 1.702, up_shift: float = 1.0, router_scale: float = 1.0, normalize: bool = True,
+                 correction: bool = True, shared: dict | None = None) -> None:
+        if not 1 <= top <= min(num_experts, hip.MOE_MAX_TOP) or num_experts > hip.MOE_MAX_EXPERTS:
+            raise ValueError(f"top {top} of {num_experts} experts: 1 <= top <= min(experts, {hip.MOE_MAX_TOP}), "
+                             f"experts <= {hip.MOE_MAX_EXPERTS}")
+        self.hidden_size, self.num_experts, self.top, self.intermediate_size = hidden_size, num_experts, top, intermediate_size
+        self.limit, self.slope, self.up_shift = limit, slope, up_shift
+        self.router_scale, self.normalize, self.has_correction = router_scale, normalize, correction
+        self.shared = CappedGLU(hidden_size=hidden_size, **shared) if shared is not None else None
+        self.router: torch.Tensor | None = None
+        self.correction: torch.Tensor | None = None
+        self.gate_up: torch.Tensor | None = None
+        self.down: torch.Tensor | None = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        E, F, H = self.num_experts, self.intermediate_size, self.hidden_size
+        specs = {"router": ParamSpec((E, H), "float32", init=(0.0, 0.2)),
+                 "gate_up": ParamSpec((E, 2 * F, H)), "down": ParamSpec((E, H, F))}
+        if self.has_correction:
+            specs["correction"] = ParamSpec((E,), "float32", init=(0.0, 0.1))
+        if self.shared is not None:
+            specs.update({f"shared_{name}": ps for name, ps in self.shared.param_specs().items()})
+        return specs
+
+    def bind(self, params) -> None:
+        own = {n: t for n, t in params.items() if not n.startswith("shared_")}
+        super().bind(own)
+        if self.shared is not None:
+            self.shared.bind({n[len("shared_"):]: t for n, t in params.items() if n.startswith("shared_")})
+
+    def widest_activation(self) -> int:
+        shared = self.shared.widest_activation() if self.shared is not None else 0
+        return max(2 * self.top * self.hidden_size, self.top * self.intermediate_size, shared)
+
+    def keep_streaming_copies(self) -> int:
+        return self.shared.keep_streaming_copies() if self.shared is not None else 0
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        experts, weights = hip.moe_route(x, self.router, self.correction, self.top, self.router_scale, self.normalize)
+        grouped = hip.moe_group(experts, self.num_experts)
+        unit = hip.moe_gemm(x, self.gate_up, grouped, x.dtype, per_token=True, glu=(self.limit, self.slope, self.up_shift))
+        rows = hip.moe_gemm(unit, self.down, grouped, torch.float32, per_token=False)
+        shared = self.shared.forward(x, ctx) if self.shared is not None else None
+        return hip.moe_combine(rows, weights, shared)

@@ -1,4 +1,4 @@
-"""RMSNorm with the residual add folded in (tinyserve_llm/model/llama.py:39-74).
+"""Norms. RMSNorm with the residual add folded in (tinyserve_llm/model/llama.py:39-74).
 
 `norm(x, residual)` returns (normalise(x + residual) * weight, x + residual): the sum, its mean
 square, the rsqrt and the scaling are 32-bit; the returned residual is the sum rounded to the
@@ -46,3 +46,42 @@ class RMSNorm(Norm):
     def made_for(self, pending) -> bool:
         """Whether `pending` is this norm, deferred (by `defer` or through `request`)."""
         return isinstance(pending, DeferredNorm) and pending.weight is self.weight and pending.eps == self.eps
+
+
+@register("norm", "dynamic_tanh")
+class DynamicTanh(Norm):
+    """tanh(alpha x) * weight + bias, element by element: no mean and no variance, so no reduction over
+    the row. alpha is one learned scalar. All of it is 32-bit; what leaves for a projection is rounded to
+    the storage type at the store. On a 32-bit residual stream the norm rides in the kernel that does the
+    stream's pending sum (`ResidualStream.take`)."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, alpha_init: float = 0.5) -> None:
+        self.hidden_size, self.alpha_init = hidden_size, alpha_init
+        self.weight: torch.Tensor | None = None
+        self.bias: torch.Tensor | None = None
+        self.alpha: torch.Tensor | None = None
+        self._f32: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {"weight": ParamSpec((self.hidden_size,), init=(1.0, 0.1)), "bias": ParamSpec((self.hidden_size,), init=(0.0, 0.02)),
+                "alpha": ParamSpec((), init=(self.alpha_init, 0.05))}
+
+    def bind(self, params) -> None:
+        super().bind(params)
+        # the kernels read 32-bit parameters (the stored type tells what the projections take)
+        self._f32 = (self.alpha.float().reshape(1).contiguous(), self.weight.float().contiguous(), self.bias.float().contiguous())
+
+    def elementwise(self) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """(alpha [1], weight, bias) in 32-bit: the norm as a kernel that works element by element takes it."""
+        return self._f32
+
+    def __call__(self, x, residual=None, rows=None):
+        if isinstance(x, ResidualStream):
+            if residual is not None:
+                raise ValueError("a residual stream carries its own sum")
+            stream, out = x.take(self, rows, self.weight.dtype)
+            return out, (None if rows is not None else stream)
+        out, total = hip.dyt(x, *self._f32, x.dtype, residual=residual, rows=rows, keep_sum=residual is not None)
+        return out, (total if residual is not None else x)
