@@ -67,3 +67,35 @@ def rugezen_configs():
     S = RugezenConfig(vocab=300, width=512, norm_eps=1e-6, residual_mult=0.45, loop_start=0, loop_stop=1, loop_times=2,
                       layers=(RugezenLayer("attention", att_u, 640), RugezenLayer("mingru", RugezenMinGRU(width=256), 768)))
     return {"P": (P, 3), "Q": (Q, 4), "R": (R, 5), "S": (S, 6)}
+
+
+def fanotar_configs():
+    """Small Fanotar configurations that differ from each other in every size and option: key/value
+    grouping, key and value head sizes (equal or not), taps of the short convolution (down to one),
+    windows (one key, shorter and longer than a page, none), query multipliers that step early or never,
+    layers that read another layer's cache through a wider or a narrower window than its owner's, dense,
+    routed (with and without a shared expert, one expert per token up to all of them) and absent
+    feed-forwards, and widths that are multiples of nothing."""
+    from tinyserve_llm_amd.config.fanotar import FanotarAttention as A, FanotarConfig, FanotarExperts as E, \
+        FanotarGatedUnit as U, FanotarLayer as L
+    a0 = A(heads=4, kv_heads=2, dim=32, vdim=48, conv=3, window=24, scale=0.3, q_temp_coef=0.4, q_temp_every=16)
+    a1 = A(heads=4, kv_heads=2, dim=32, vdim=48, conv=2, window=50, scale=0.2, q_temp_coef=0.25, q_temp_every=7, kv_from=0)
+    a2 = A(heads=6, kv_heads=1, dim=24, vdim=8, conv=1, window=0, scale=0.35, q_temp_coef=0.0, q_temp_every=1)
+    P = FanotarConfig(vocab=200, width=80, norm_eps=1e-6, embedding_scale=7.0, layers=(
+        L(a0, U(ff=96, limit=1.5)), L(a1, E(experts=6, top=3, scale=1.7, expert=U(40, 1.0), shared=U(24, 2.0))), L(a2, None)))
+    b0 = A(heads=2, kv_heads=2, dim=16, vdim=16, conv=5, window=1, scale=0.25, q_temp_coef=1.0, q_temp_every=3)
+    b1 = A(heads=2, kv_heads=2, dim=16, vdim=16, conv=2, window=70, scale=0.4, q_temp_coef=0.3, q_temp_every=100)
+    b2 = A(heads=2, kv_heads=2, dim=16, vdim=16, conv=4, window=9, scale=0.4, q_temp_coef=0.3, q_temp_every=100, kv_from=1)
+    Q = FanotarConfig(vocab=131, width=48, norm_eps=1e-4, embedding_scale=1.0, layers=(
+        L(b0, E(experts=4, top=1, scale=1.0, expert=U(20, 3.0), shared=None)), L(b1, U(64, 0.7)), L(b2, U(40, 2.5)),
+        L(b2, E(experts=3, top=3, scale=0.6, expert=U(12, 1.2), shared=U(8, 1.0)))))
+    # sizes that are multiples of nothing in particular: no kernel's fast path takes them
+    c0 = A(heads=3, kv_heads=1, dim=20, vdim=12, conv=4, window=7, scale=0.3, q_temp_coef=0.5, q_temp_every=2)
+    R = FanotarConfig(vocab=77, width=99, norm_eps=1e-5, embedding_scale=3.5, layers=(
+        L(c0, E(experts=5, top=2, scale=2.2, expert=U(17, 2.0), shared=U(9, 0.5))), L(c0, U(52, 1.0))))
+    # a width that the weight-streaming kernels take, heads of a matrix-core size, experts in tiles of several rows
+    d0 = A(heads=8, kv_heads=2, dim=64, vdim=64, conv=4, window=33, scale=0.11, q_temp_coef=0.2, q_temp_every=32)
+    d1 = A(heads=8, kv_heads=2, dim=64, vdim=64, conv=4, window=130, scale=0.11, q_temp_coef=0.2, q_temp_every=32, kv_from=0)
+    S = FanotarConfig(vocab=300, width=512, norm_eps=1e-6, embedding_scale=12.0, layers=(
+        L(d0, E(experts=8, top=2, scale=1.5, expert=U(128, 2.0), shared=U(256, 1.0))), L(d1, U(640, 2.0))))
+    return {"P": (P, 3), "Q": (Q, 4), "R": (R, 5), "S": (S, 6)}

@@ -113,9 +113,10 @@ class PlainFanotar:
         pos = torch.arange(n)
         q = short_convolution(h @ self.w[p + "q"].T, self.w[p + "q.conv"]).view(n, m["heads"], m["dim"])
         q = unit_rms(q, self.eps) * self.w[p + "q.norm"]
-        q = q * query_multiplier(pos.to(self.dtype), m["q_temp"]["coef"], m["q_temp"]["every"])[:, None, None]
+        if m.get("q_temp"):
+            q = q * query_multiplier(pos.to(self.dtype), m["q_temp"]["coef"], m["q_temp"]["every"])[:, None, None]
         o = sloped_sink_attention(q, kv[0], kv[1], pos, m["scale"], distance_slopes(m["heads"]), self.w[p + "sink"],
-                                  m["mask"]["size"])
+                                  m["mask"]["size"] if m.get("mask") else 0)
         gate = torch.sigmoid(h @ self.w[p + "g"].T)
         return (o.reshape(n, -1) * gate) @ self.w[p + "o"].T
 
