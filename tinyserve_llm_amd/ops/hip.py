@@ -1759,7 +1759,8 @@ def paged_attention_general(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     _run("paged_attention_general", library().ts_paged_attention_general(
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
         T, nh, nkv, hd, vd, k_cache.shape[1], *k_cache.stride()[:3], *v_cache.stride(), block_tables.shape[1],
-        float(scale), float(softcap), int(sink), int(window), _code(q.dtype), _page_run(pages_per_entry), _stream()))
+        float(scale), float(softcap), int(sink), int(window), _code(q.dtype), _page_run(pages_per_entry), None, None, None, 0,
+        _stream()))
     return out
 
 
