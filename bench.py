@@ -22,6 +22,14 @@ tokens/s at batch 1, 8 and 64 through the whole engine, and kernel by kernel the
 norms, the feed-forward's activation) with the bytes or operations each has to move and what share of
 the machine's peak that comes to. One JSON line.
 
+    python bench.py --fanotar [--shape 1b|3b] [--layers L]
+
+measures the Fanotar decoder (dynamic-tanh norms around every part on a 32-bit stream, attention behind a
+short convolution with distance slopes, learned sinks, a window and an output gate, every fourth layer
+reading its neighbour's cache, capped gated feed-forward, dense and as a mixture of experts in turn) beside
+the Rugezen decoder, the closest of the engine's models, at equal layer sizes and equal active parameters
+per token, in the same way: whole-engine throughput and the like kernels side by side. One JSON line.
+
     python bench.py --scenario requests-3b | chunked-8b [--layers L]
 
 runs a whole workload through `LLM.generate` instead and prints one JSON line of its own: many
@@ -340,6 +348,253 @@ def designs(args) -> int:
     return 0
 
 
+def fanotar(args) -> int:
+    """The Fanotar decoder beside the Rugezen decoder at the layer sizes of `--shape`: whole-engine
+    throughput, and the like kernels of the two side by side. One JSON line."""
+    import torch
+
+    from tinyserve_llm_amd.config.fanotar import FanotarAttention, FanotarConfig, FanotarExperts, FanotarGatedUnit, FanotarLayer
+    from tinyserve_llm_amd.config.rugezen import RugezenAttention, RugezenConfig, RugezenLayer
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.loading import random_model
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    from tinyserve_llm_amd.ops import hip
+    from tinyserve_llm_amd.parts.base import StepContext
+    from tinyserve_llm_amd.parts.linear import linear
+
+    sizes = SHAPES[args.shape]
+    sh = sizes["shape"]
+    layers = args.layers or sizes["layers_full"]
+    hidden, nh, nkv, hd, inter, vocab = (sh["hidden_size"], sh["num_attention_heads"], sh["num_key_value_heads"], sh["head_dim"],
+                                         sh["intermediate_size"], sh["vocab_size"])
+    window, taps, experts, top = 1024, 4, 16, 4
+    eff, sff = inter // 8, inter // 2                 # four experts of an eighth and a shared half: one dense width per token
+    ratt = RugezenAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, rot_dims=hd // 2, rot_base=1.0e6, scale=hd ** -0.5, softcap=30.0)
+    rug = RugezenConfig(vocab=vocab, width=hidden, norm_eps=1e-6, residual_mult=0.6,
+                        layers=tuple(RugezenLayer("attention", ratt, 3 * inter // 2) for _ in range(layers)))
+
+    def fan_layer(i):
+        att = FanotarAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, conv=taps, window=window, scale=hd ** -0.5, q_temp_coef=0.1,
+                               q_temp_every=1024, kv_from=i - 1 if i % 4 == 3 else None)
+        dense = FanotarGatedUnit(inter, 7.0)
+        moe = FanotarExperts(experts=experts, top=top, scale=2.5, expert=FanotarGatedUnit(eff, 7.0), shared=FanotarGatedUnit(sff, 7.0))
+        return FanotarLayer(att, moe if i % 2 else dense)
+    fan = FanotarConfig(vocab=vocab, width=hidden, norm_eps=1e-6, embedding_scale=float(hidden) ** 0.5,
+                        layers=tuple(fan_layer(i) for i in range(layers)))
+    prompt_len = args.context
+    max_model_len = max(MAX_MODEL_LEN, prompt_len + 1024)
+    rng = random.Random(0)
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def whole_engine(config) -> dict:
+        model = random_model(config, 0, torch.bfloat16, "cuda:0")
+        import math
+        out = {"parameters": sum(math.prod(ps.shape) for name, ps in model.param_specs().items() if name.startswith("layers."))}
+
+        def engine(batch):
+            pages = batch * -(-max_model_len // PAGE) + 2
+            sc = SchedulerConfig(max_model_len=max_model_len, max_num_seqs=batch,
+                                 max_num_batched_tokens=max(prompt_len, batch + 1) + batch, watermark=0.0)
+            return LLM(None, sc, CacheConfig(block_size=PAGE, caching=False), dtype=torch.bfloat16, num_blocks=pages, seed=0,
+                       model=model)
+        llm = engine(1)
+        times = []
+        for r in range(3):
+            llm.add_request([rng.randrange(vocab) for _ in range(prompt_len)], SamplingParams(max_tokens=1, temperature=0.0, ignore_eos=True))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            llm.step()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        out["prefill_tok_s"] = prompt_len / min(times[1:])
+        del llm
+        for batch in (1, 8, 64):
+            llm = engine(batch)
+            sp = SamplingParams(max_tokens=max_model_len - prompt_len, temperature=0.0, ignore_eos=True)
+            for _ in range(batch):
+                llm.add_request([rng.randrange(vocab) for _ in range(prompt_len)], sp)
+            while any(q.in_prefill or not q.output_token_ids for q in llm.scheduler.running + llm.scheduler.waiting):
+                llm.step()
+            for _ in range(6):
+                llm.step()
+            steps = 32
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                llm.step()
+            torch.cuda.synchronize()
+            out[f"decode_b{batch}_tok_s"] = batch * steps / (time.perf_counter() - t0)
+            del llm
+        del model
+        torch.cuda.empty_cache()
+        return out
+
+    sweep = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
+    overhead = []
+
+    def replayed(fn, reps: int) -> float:
+        fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            kept = fn()
+        best = float("inf")
+        for _ in range(reps):
+            sweep.sum()
+            begin.record()
+            graph.replay()
+            end.record()
+            end.synchronize()
+            best = min(best, 1e3 * begin.elapsed_time(end))
+        del kept, graph
+        return best
+
+    def timed(fn, reps: int = 5) -> float:
+        """Microseconds of the best replay of `fn` recorded into a graph, each after a sweep of the caches,
+        less what the replay of a graph of one tiny kernel takes."""
+        if not overhead:
+            tiny = torch.zeros(64, dtype=torch.int32, device="cuda")
+            overhead.append(replayed(lambda: tiny.add_(1), reps))
+        return max(replayed(fn, reps) - overhead[0], 1e-3)
+
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    bf = torch.bfloat16
+
+    def context(starts, counts, pool_page):
+        positions, seq_of, cu, tables = [], [], [0], []
+        per = -(-max(a + b for a, b in zip(starts, counts)) // PAGE)
+        for i, (s0, n) in enumerate(zip(starts, counts)):
+            positions += list(range(s0, s0 + n))
+            seq_of += [i] * n
+            cu.append(cu[-1] + n)
+            tables.append(list(range(i * per, (i + 1) * per)))
+        ends = [a + b for a, b in zip(starts, counts)]
+        slots = dev([tables[i][p // PAGE] * PAGE + p % PAGE for i, p in zip(seq_of, positions)])
+        ctx = StepContext(num_tokens=len(positions), num_seqs=len(starts), token_ids=dev([0] * len(positions)), positions=dev(positions),
+                          seq_of_token=dev(seq_of), cu_seqlens=dev(cu), context_lens=dev(ends), state_slots=dev(list(range(len(starts)))),
+                          slot_mapping=[slots], block_tables=[dev(tables)], host_cu_seqlens=cu, host_starts=list(starts),
+                          host_context_lens=ends, host_state_slots=list(range(len(starts))), page_size=PAGE)
+        return ctx, slots, len(starts) * per * (PAGE // pool_page)
+
+    def kernel_pairs() -> dict:
+        pairs = {}
+        pool_page = 32
+        peaks = hip.measure_peaks()
+        read_peak, mfma_peak = peaks["read_GBps"] * 1e9, peaks["mfma_bf16_TFLOPs"] * 1e12
+        slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / nh) for h in range(nh)], device="cuda")
+        sinks = torch.randn(nh, device="cuda")
+        for label, starts, counts in (("prompt portion", [0], [prompt_len]), ("decoded tokens, batch 64", [prompt_len] * 64, [1] * 64)):
+            ctx, slots, pages = context(starts, counts, pool_page)
+            T = ctx.num_tokens
+            k = torch.randn(pages, nkv, pool_page, hd, device="cuda").to(bf).permute(0, 2, 1, 3)
+            v = torch.randn(pages, nkv, hd, pool_page, device="cuda").to(bf).permute(0, 3, 1, 2)
+            q = torch.randn(T, nh, hd, device="cuda").to(bf)
+            gate = torch.randn(T, nh * hd, device="cuda")
+            seen = lambda s0, n, w: sum(min(p + 1, w) if w else p + 1 for p in range(s0, s0 + n))
+            keys_r = sum(seen(s0, n, 0) for s0, n in zip(starts, counts))
+            keys_f = sum(seen(s0, n, window) for s0, n in zip(starts, counts))
+            us_r = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5, softcap=30.0, sink=True))
+            us_f = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5, window, sinks=sinks, slopes=slopes, gate=gate))
+            us_f0 = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5, window, sinks=sinks, slopes=slopes))
+            if T > 64:
+                fr, ff_ = 4 * nh * hd * keys_r, 4 * nh * hd * keys_f
+                pairs[f"attention, {label}"] = {"rugezen_us": us_r, "fanotar_us": us_f, "fanotar_us_without_gate": us_f0,
+                                                "rugezen_flops": fr, "fanotar_flops": ff_,
+                                                "rugezen_frac_of_mfma": fr / us_r * 1e6 / mfma_peak,
+                                                "fanotar_frac_of_mfma": ff_ / us_f * 1e6 / mfma_peak}
+            else:
+                br = sum(s0 + n for s0, n in zip(starts, counts)) * 2 * nkv * hd * 2
+                bfan = sum(min(s0 + n, window) for s0, n in zip(starts, counts)) * 2 * nkv * hd * 2
+                pairs[f"attention, {label}"] = {"rugezen_us": us_r, "fanotar_us": us_f, "fanotar_us_without_gate": us_f0,
+                                                "rugezen_bytes": br, "fanotar_bytes": bfan,
+                                                "rugezen_frac_of_read": br / us_r * 1e6 / read_peak,
+                                                "fanotar_frac_of_read": bfan / us_f * 1e6 / read_peak}
+            # between projection and cache: rotation and three head norms, against convolution, two head norms and the state
+            row = (nh + 2 * nkv) * hd
+            freqs = torch.rand(hd // 4, dtype=torch.float64, device="cuda")
+            qkv32 = torch.randn(T, row + nh * hd, device="cuda")
+            plain32 = qkv32[:, :row].contiguous()
+            conv = torch.randn(row, taps, device="cuda")
+            state = torch.zeros(len(starts), taps - 1, row, device="cuda")
+            nw = torch.ones(hd, device="cuda")
+            us_r = timed(lambda: hip.qkv_finish(plain32, freqs, ctx.positions, slots, k, v, nh, nkv, hd, hd, bf, qk_norm_eps=1e-5, v_norm_eps=1e-5))
+
+            def finish():
+                out = hip.conv_finish(qkv32, conv, state, ctx, slots, k, v, nh, nkv, hd, hd, bf, q_norm=nw, k_norm=nw, eps=1e-5,
+                                      temp_coef=0.1, temp_every=1024)
+                hip.conv_state_update(state, qkv32, ctx)
+                return out
+            us_f = timed(finish)
+            nbytes = T * row * (4 + 2)
+            pairs[f"between projection and cache, {label}"] = {"rugezen_us": us_r, "fanotar_us": us_f, "bytes": nbytes,
+                                                               "rugezen_frac_of_read": nbytes / us_r * 1e6 / read_peak,
+                                                               "fanotar_frac_of_read": nbytes / us_f * 1e6 / read_peak}
+            # the stream's sum and norms: two branches and two RMS norms once a layer, against one branch through its norm and
+            # one norm out, twice a layer
+            w16 = torch.ones(hidden, device="cuda").to(bf)
+            x32, a32, b32 = (torch.randn(T, hidden, device="cuda") for _ in range(3))
+            norm = (torch.full((1,), 0.5, device="cuda"), torch.ones(hidden, device="cuda"), torch.zeros(hidden, device="cuda"))
+            us_r = timed(lambda: hip.stream_update_norm(x32, a32, b32, None, 0.6, (w16, w16), 1e-6, out_dtype=bf))
+            us_f = timed(lambda: hip.dyt_stream(x32, a32, norm, norm, bf))
+            bytes_r, bytes_f = T * hidden * (4 * 4 + 2 * 2), T * hidden * (3 * 4 + 2)
+            pairs[f"stream sum and norms, {label}"] = {"rugezen_us": us_r, "fanotar_us": us_f, "rugezen_bytes": bytes_r, "fanotar_bytes": bytes_f,
+                                                       "fanotar_launches_a_layer": 2,
+                                                       "rugezen_frac_of_read": bytes_r / us_r * 1e6 / read_peak,
+                                                       "fanotar_frac_of_read": bytes_f / us_f * 1e6 / read_peak}
+            rff = 3 * inter // 2
+            up, bias, gu = torch.randn(T, rff, device="cuda"), torch.randn(rff, device="cuda").to(bf), torch.randn(T, 2 * inter, device="cuda")
+            us_r = timed(lambda: hip.bias_activation(up, bias, "relu2", bf))
+            us_f = timed(lambda: hip.capped_glu(gu, 7.0, 1.702, 1.0, bf))
+            bytes_r, bytes_f = T * rff * (4 + 2), T * inter * (2 * 4 + 2)
+            pairs[f"feed-forward activation, {label}"] = {"rugezen_us": us_r, "fanotar_us": us_f, "rugezen_bytes": bytes_r, "fanotar_bytes": bytes_f,
+                                                          "rugezen_frac_of_read": bytes_r / us_r * 1e6 / read_peak,
+                                                          "fanotar_frac_of_read": bytes_f / us_f * 1e6 / read_peak}
+            # the experts' two products (routing and grouping beside them) against a dense feed-forward's two of the same
+            # operations per token through `linear`
+            x16 = torch.randn(T, hidden, device="cuda").to(bf)
+            router, corr = torch.randn(experts, hidden, device="cuda") * 0.02, torch.zeros(experts, device="cuda")
+            wgu = (torch.randn(experts, 2 * eff, hidden, device="cuda") * 0.02).to(bf)
+            wd = (torch.randn(experts, hidden, eff, device="cuda") * 0.02).to(bf)
+            dgu = (torch.randn(2 * top * eff, hidden, device="cuda") * 0.02).to(bf)
+            dd = (torch.randn(hidden, top * eff, device="cuda") * 0.02).to(bf)
+            ids, wts = hip.moe_route(x16, router, corr, top, 2.5)
+            tile_rows = hip.moe_tile_rows(ids.numel(), experts, bf, (hidden, eff))
+            grouped = hip.moe_group(ids, experts, tile_rows)
+            us_route = timed(lambda: (hip.moe_route(x16, router, corr, top, 2.5), hip.moe_group(ids, experts, tile_rows)))
+
+            def products():
+                unit = hip.moe_gemm(x16, wgu, grouped, bf, per_token=True, glu=(7.0, 1.702, 1.0))
+                return hip.moe_combine(hip.moe_gemm(unit, wd, grouped, torch.float32, per_token=False), wts)
+
+            def dense():
+                unit = hip.capped_glu(linear(x16, dgu, out_dtype=torch.float32), 7.0, 1.702, 1.0, bf)
+                return linear(unit, dd, out_dtype=torch.float32)
+            us_f, us_d = timed(products), timed(dense)
+            flops = 2 * T * top * 3 * eff * hidden
+            touched = min(experts, T * top) * 3 * eff * hidden * 2
+            rec = {"fanotar_us": us_f, "dense_of_equal_work_us": us_d, "routing_and_grouping_us": us_route, "flops": flops,
+                   "tile_rows": tile_rows}
+            if T > 64:
+                rec.update(fanotar_frac_of_mfma=flops / us_f * 1e6 / mfma_peak, dense_frac_of_mfma=flops / us_d * 1e6 / mfma_peak)
+            else:
+                rec.update(expert_bytes=touched, fanotar_frac_of_read=touched / us_f * 1e6 / read_peak,
+                           dense_bytes=top * 3 * eff * hidden * 2, dense_frac_of_read=top * 3 * eff * hidden * 2 / us_d * 1e6 / read_peak)
+            pairs[f"experts' products, {label}"] = rec
+        pairs["peaks"] = {"read_GBps": read_peak / 1e9, "mfma_bf16_TFLOPs": mfma_peak / 1e12}
+        return pairs
+
+    record = {"designs": {"rugezen": whole_engine(rug), "fanotar": whole_engine(fan)}, "kernels": kernel_pairs(),
+              "config": {"shape": args.shape, "layers": layers, "hidden": hidden, "heads": nh, "kv_heads": nkv, "head_dim": hd,
+                         "rugezen_ff": 3 * inter // 2, "fanotar_dense_ff": inter, "fanotar_experts": experts, "fanotar_top": top,
+                         "fanotar_expert_ff": eff, "fanotar_shared_ff": sff, "fanotar_window": window, "fanotar_conv_taps": taps,
+                         "fanotar_layers": "dense and routed feed-forward in turn; every fourth layer reads the cache of the one before",
+                         "vocab": vocab, "context": prompt_len, "dtype": "bf16",
+                         "data": "synthetic uniform token ids, random weights"}}
+    print(json.dumps(record))
+    return 0
+
+
 def kernel_classes(llm, config, batch: int, reps: int = 5) -> dict:
     """Times one decode step's kernels by class. An eager step (no graph) is run once with every
     launch of the engine's kernel module noted down with its operands; then each class's launches
@@ -467,6 +722,9 @@ def main() -> int:
     ap.add_argument("--designs", action="store_true",
                     help="measure the Rugezen decoder beside the Llama decoder at the layer sizes of --shape: whole-engine "
                          "throughput and the like kernels side by side; one JSON line")
+    ap.add_argument("--fanotar", action="store_true",
+                    help="measure the Fanotar decoder beside the Rugezen decoder at the layer sizes of --shape: whole-engine "
+                         "throughput and the like kernels side by side; one JSON line")
     ap.add_argument("--kernel-classes", action="store_true",
                     help="time one decode step's kernels class by class (bytes, microseconds, GB/s) and exit")
     ap.add_argument("--peaks", action="store_true",
@@ -492,6 +750,8 @@ def main() -> int:
         return scenario(args.scenario, args.layers, args.dtype)
     if args.designs:
         return designs(args)
+    if args.fanotar:
+        return fanotar(args)
     sizes = SHAPES[args.shape]
     full_layers = sizes["layers_full"]
     args.layers = args.layers or full_layers

@@ -32,7 +32,8 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
                         const int32_t* __restrict__ block_tables, const int32_t* __restrict__ seq_of_token,
                         const int32_t* __restrict__ positions, int nh, int G, int page_size, int page_shift, int page_run,
                         int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
-                        int num_splits, int chunk, float scale2, int window, float cap_in, float cap_out, int sink) {
+                        int num_splits, int chunk, float scale2, int window, float cap_in, float cap_out, int sink,
+                        const float* __restrict__ sinks, const float* __restrict__ slopes) {
   constexpr int NC = HD / 32;    // 32-dimension pieces of a key row (one 16-byte load per lane each)
   constexpr int NDB = HD / 16;   // 16-dimension blocks of the output
   ts_fetch_arguments<GENERAL ? 176 : 164>();     // (nine pointers, five numbers, six strides, four more numbers and the scale; the caps and the sink)
@@ -75,7 +76,9 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
   if (kend > pos + 1) kend = pos + 1;
   int kb = (k0 > (lo & ~31) ? k0 : (lo & ~31)) + 32 * wave;
 #define TS_LOAD(T, KB) load_tile<HD>(T, KB, r, g, lo, pos, kvh, table, pm, k_cache, v_cache, kp, ks, kh, vp, vh, vd)
-#define TS_USE(T, KB) use_tile_auto<HD, GENERAL>(T, KB, r, g, lo, pos, pos, lo, qreg, scale2, m, l, o, cap_in, cap_out)
+  // (the general variant: this row's head's penalty per position of distance, in the scores' units before scale2)
+  const float slope = (GENERAL && slopes && r < G) ? slopes[kvh * G + r] * (1.44269504088896340736f / scale2) : 0.f;
+#define TS_USE(T, KB) use_tile_auto<HD, GENERAL>(T, KB, r, g, lo, pos, pos, lo, qreg, scale2, m, l, o, cap_in, cap_out, slope)
   if (ONE) {
     if (kb < kend) {
       KVTile<HD> A;
@@ -125,7 +128,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
       L = fmaf(wl[w * 16 + head], wgt, L);
     }
     if (num_splits == 1) {                  // the whole context was this workgroup's: position `pos` is always visible
-      if (GENERAL && sink) L += fast_exp2(-M);
+      if (GENERAL && sink) L += fast_exp2((sinks ? sinks[kvh * G + head] * 1.44269504088896340736f : 0.f) - M);
       out[((int64_t)t * nh + (int64_t)kvh * G + head) * HD + d] = f2bf(acc / L);
     } else {
       const int64_t row = ((int64_t)t * nh + (int64_t)kvh * G + head) * num_splits + split;
@@ -143,7 +146,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
 __global__ void __launch_bounds__(TS_WAVE)
 attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                            const float* __restrict__ part_ml, const int32_t* __restrict__ positions, int nh, int hd,
-                           int num_splits, int chunk, int window, int sink) {
+                           int num_splits, int chunk, int window, int sink, const float* __restrict__ sinks) {
   __shared__ float wgt[COMBINE_MAX_SPLITS];
   const int t = blockIdx.x / nh, lane = threadIdx.x;
   const int64_t th = blockIdx.x;
@@ -161,7 +164,8 @@ attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ p
     L += ml[2 * s + 1] * w;
   }
   L = wave_sum(L);
-  if (sink) L += fast_exp2(-M);           // the sink's score is 0
+  // the sink's score is 0, or its head's learned one
+  if (sink) L += fast_exp2((sinks ? sinks[blockIdx.x % nh] * 1.44269504088896340736f : 0.f) - M);
   wave_sync();
   const float inv = 1.0f / L;
   const float* po = part_o + (th * num_splits + s0) * hd;
@@ -185,10 +189,10 @@ extern "C" int ts_attention_combine(void* out, const float* part_o, const float*
 // The combining kernel alone, for the prefill kernel's split walks (declared in attention_mfma.h).
 int ts_launch_attention_combine(void* out, const float* part_o, const float* part_ml, const int32_t* positions,
                                 int num_tokens, int nh, int hd, int num_splits, int chunk, int window,
-                                hipStream_t stream, int sink) {
+                                hipStream_t stream, int sink, const float* sinks) {
   if (num_splits > COMBINE_MAX_SPLITS) return TS_BAD_SHAPE;
   attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,
-                                                                      num_splits, chunk, window, sink);
+                                                                      num_splits, chunk, window, sink, sinks);
   return ts_check_launch();
 }
 
@@ -206,7 +210,7 @@ static int launch_decode(void* out, float* part_o, float* part_ml, const void* q
                          int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
                          int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits, int chunk,
                          int waves, float scale, int window, int page_run, int combine, bool general, float softcap, int sink,
-                         hipStream_t stream) {
+                         const float* sinks, const float* slopes, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || num_splits <= 0 || page_run < 0 || page_run > 16)
     return TS_BAD_SHAPE;
@@ -235,7 +239,7 @@ static int launch_decode(void* out, float* part_o, float* part_ml, const void* q
   attn_decode_mfma_kernel<HH, ON, GG><<<grid, waves * TS_WAVE, smem, stream>>>(                                 \
       (bf16_t*)out, part_o, part_ml, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,          \
       block_tables, seq_of_token, positions, nh, G, page_size, page_shift, page_run, kp, ks, kh, vp, vh, vd, max_blocks,  \
-      num_splits, chunk, scale2, window, cap_in, cap_out, sink)
+      num_splits, chunk, scale2, window, cap_in, cap_out, sink, sinks, slopes)
 #define TS_DEC1(HH, ON) if (general) TS_DEC2(HH, ON, true); else TS_DEC2(HH, ON, false)
 #define TS_DEC(HH) if (chunk == 32 * waves) { TS_DEC1(HH, true); } else { TS_DEC1(HH, false); }
   switch (hd) {
@@ -251,7 +255,8 @@ static int launch_decode(void* out, float* part_o, float* part_ml, const void* q
   int rc = ts_check_launch();
   if (rc || num_splits == 1 || !combine) return rc;     // (combine 0: the caller's next kernel reads the parts itself)
   attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,
-                                                                      num_splits, chunk, window, general ? sink : 0);
+                                                                      num_splits, chunk, window, general ? sink : 0,
+                                                                      general ? sinks : nullptr);
   return ts_check_launch();
 }
 
@@ -263,20 +268,21 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
                                          int waves, float scale, int window, int page_run, int combine, hipStream_t stream) {
   return launch_decode(out, part_o, part_ml, q, k_cache, v_cache, block_tables, seq_of_token, positions, num_tokens, nh, nkv, hd,
                        page_size, kp, ks, kh, vp, vh, vd, max_blocks, num_splits, chunk, waves, scale, window, page_run, combine,
-                       false, 0.f, 0, stream);
+                       false, 0.f, 0, nullptr, nullptr, stream);
 }
 
 // The same with capped scores (softcap > 0: cap * tanh(score / cap)), a sink (one more in the softmax's
-// denominator) and weights carried in two bfloat16 terms; always combines.
+// denominator; `sinks`, float [nh], if given: exp(sinks[head]) more instead), a penalty of slopes[head] (float [nh],
+// if given) per position of distance taken off every score, and weights carried in two bfloat16 terms; always combines.
 extern "C" int ts_paged_attention_decode_general(void* out, float* part_o, float* part_ml, const void* q, const void* k_cache,
                                                  const void* v_cache, const int32_t* block_tables,
                                                  const int32_t* seq_of_token, const int32_t* positions, int num_tokens,
                                                  int nh, int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
                                                  int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits,
                                                  int chunk, int waves, float scale, int window, int page_run, float softcap,
-                                                 int sink, hipStream_t stream) {
+                                                 int sink, const float* sinks, const float* slopes, hipStream_t stream) {
   if (softcap < 0.f) return TS_BAD_SHAPE;
   return launch_decode(out, part_o, part_ml, q, k_cache, v_cache, block_tables, seq_of_token, positions, num_tokens, nh, nkv, hd,
                        page_size, kp, ks, kh, vp, vh, vd, max_blocks, num_splits, chunk, waves, scale, window, page_run, 1,
-                       true, softcap, sink, stream);
+                       true, softcap, sink || sinks, sinks, slopes, stream);
 }

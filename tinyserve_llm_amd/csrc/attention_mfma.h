@@ -143,12 +143,14 @@ static __device__ __forceinline__ void tile_scores(const uint4 (&k)[2][HD / 32],
 // (the caller has checked).
 // GENERAL: the variant for mixers with capped scores and weights that must not lose their 32 bits. With cap_in
 // != 0 a score becomes cap_out * tanh(score * cap_in) first (cap_in = scale / cap, cap_out = cap * log2 e, and
-// scale2 = 1); and the weights enter the products as two bfloat16 terms, P = hi + lo with lo = P - hi rounded
+// scale2 = 1); `slope` times the distance between the row's position and the key's is taken off every score (after
+// the cap); and the weights enter the products as two bfloat16 terms, P = hi + lo with lo = P - hi rounded
 // again, which carries 16 bits of their mantissa (the plain variant rounds P to 8).
 template <int HD, bool MASKED, typename L, bool GENERAL = false>
 static __device__ __forceinline__ void tile_softmax_values(float4_t (&s)[2], const uint4 (&v)[HD / 16], bool vok, int kb, int r,
                                                            int g, int lo, int pos, float scale2, float& m, L& l,
-                                                           float4_t (&o)[HD / 16], float cap_in = 0.f, float cap_out = 0.f) {
+                                                           float4_t (&o)[HD / 16], float cap_in = 0.f, float cap_out = 0.f,
+                                                           float slope = 0.f) {
   constexpr int NDB = HD / 16;
   constexpr bool SUMS_BY_MFMA = std::is_same<L, float4_t>::value;
   if constexpr (GENERAL) {
@@ -161,6 +163,14 @@ static __device__ __forceinline__ void tile_softmax_values(float4_t (&s)[2], con
           const float e = fast_exp2(s[tau][j] * (cap_in * 2.88539008177792681472f));
           s[tau][j] = cap_out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e));
         }
+    }
+    if (slope != 0.f) {
+      // a penalty on distance: `slope` (in the scores' units before scale2, this lane's row's) per position between
+      // the row's own and the key's
+#pragma unroll
+      for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[tau][j] -= slope * (float)max(pos - (kb + 8 * g + 4 * tau + j), 0);
     }
   }
   // this lane: row r, keys kb + 8 g + 4 tau + j
@@ -235,10 +245,11 @@ static __device__ __forceinline__ void tile_softmax_values(float4_t (&s)[2], con
 template <int HD, bool MASKED, typename L, bool GENERAL = false>
 static __device__ __forceinline__ void use_tile(const KVTile<HD>& T, int kb, int r, int g, int lo, int pos,
                                                 const uint4 (&qreg)[HD / 32], float scale2, float& m, L& l,
-                                                float4_t (&o)[HD / 16], float cap_in = 0.f, float cap_out = 0.f) {
+                                                float4_t (&o)[HD / 16], float cap_in = 0.f, float cap_out = 0.f,
+                                                float slope = 0.f) {
   float4_t s[2];
   tile_scores<HD>(T.k, qreg, s);
-  tile_softmax_values<HD, MASKED, L, GENERAL>(s, T.v, T.vok, kb, r, g, lo, pos, scale2, m, l, o, cap_in, cap_out);
+  tile_softmax_values<HD, MASKED, L, GENERAL>(s, T.v, T.vok, kb, r, g, lo, pos, scale2, m, l, o, cap_in, cap_out, slope);
 }
 
 // The same, choosing the variant: `pmin` and `lomax` are the smallest position and the largest
@@ -247,15 +258,15 @@ template <int HD, bool GENERAL = false>
 static __device__ __forceinline__ void use_tile_auto(const KVTile<HD>& T, int kb, int r, int g, int lo, int pos,
                                                      int pmin, int lomax, const uint4 (&qreg)[HD / 32], float scale2,
                                                      float& m, float& l, float4_t (&o)[HD / 16], float cap_in = 0.f,
-                                                     float cap_out = 0.f) {
-  if (kb + 31 <= pmin && kb >= lomax) use_tile<HD, false, float, GENERAL>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o, cap_in, cap_out);
-  else use_tile<HD, true, float, GENERAL>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o, cap_in, cap_out);
+                                                     float cap_out = 0.f, float slope = 0.f) {
+  if (kb + 31 <= pmin && kb >= lomax) use_tile<HD, false, float, GENERAL>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o, cap_in, cap_out, slope);
+  else use_tile<HD, true, float, GENERAL>(T, kb, r, g, lo, pos, qreg, scale2, m, l, o, cap_in, cap_out, slope);
 }
 
 // out[t, h, :] from the chunks' partial results part_o [tokens, nh, num_splits, hd] and part_ml
 // [tokens, nh, num_splits, 2] (reference maximum in units of log2, sum), over the chunks that hold
 // keys visible from positions[t] (defined in attention_decode.hip). `sink`: the softmax has one more in its
-// denominator (a key of score 0 without a value), added once, here.
+// denominator (a key of score 0 without a value, or of score sinks[head] where `sinks` is given), added once, here.
 int ts_launch_attention_combine(void* out, const float* part_o, const float* part_ml, const int32_t* positions,
                                 int num_tokens, int nh, int hd, int num_splits, int chunk, int window,
-                                hipStream_t stream, int sink = 0);
+                                hipStream_t stream, int sink = 0, const float* sinks = nullptr);

@@ -50,7 +50,8 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
              const int32_t* __restrict__ positions, const int32_t* __restrict__ tiles, int nh, int G, int page_size,
              int page_shift, int page_run, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
              float scale2, int window, float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits,
-             int chunk, int split, float cap_in, float cap_out, int sink) {
+             int chunk, int split, float cap_in, float cap_out, int sink, const float* __restrict__ sinks,
+             const float* __restrict__ slopes) {
   constexpr int NC = HD / 32, NDB = HD / 16;   // operand registers of a 32-key step: 2 NC of K, NDB of V
   auto& stage = lds.stage;
   auto& wg_range = lds.range;
@@ -63,6 +64,8 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
 
   // lane r carries row r of each of its wave's score tiles: token tk[j], head r % G of the group
   const int hh = r % G;
+  // (the general variant: this row's head's penalty per position of distance, in the scores' units before scale2)
+  const float slope = (GENERAL && slopes) ? slopes[kvh * G + hh] * (1.44269504088896340736f / scale2) : 0.f;
   int pos[RT], lo[RT], tk[RT];
   int pmax = -1, lmin = 0x7fffffff;
 #pragma unroll
@@ -263,9 +266,9 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
         if constexpr (decltype(masked)::value) {
           // a step wholly beyond the tile's last position, or wholly before all its windows, has nothing for it
           if (kb <= tile_pmax[j] && kb + 31 >= tile_lomin[j])
-            use_tile<HD, true, float4_t, GENERAL>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j], cap_in, cap_out);
+            use_tile<HD, true, float4_t, GENERAL>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j], cap_in, cap_out, slope);
         } else {
-          use_tile<HD, false, float4_t, GENERAL>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j], cap_in, cap_out);
+          use_tile<HD, false, float4_t, GENERAL>(T, kb, r, g, lo[j], pos[j], qreg[j], scale2, m[j], l[j], o[j], cap_in, cap_out, slope);
         }
       }
       __syncthreads();
@@ -294,7 +297,9 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
       float lj = l[j][i];
       const int rtk = (wave * RT + j) * tpt + row / G, rhh = row % G;
       const float mj = __shfl(m[j], row, TS_WAVE);       // the row's reference maximum (lane `row` holds it)
-      if (GENERAL && sink && num_splits == 1 && lj > 0.f) lj += fast_exp2(-mj);   // the sink's score is 0
+      // the sink's score is 0, or its head's learned one
+      if (GENERAL && sink && num_splits == 1 && lj > 0.f)
+        lj += fast_exp2((sinks ? sinks[kvh * G + rhh] * 1.44269504088896340736f : 0.f) - mj);
       if (num_splits > 1) {
         // the chunk's share of the row, not normalised: sums, and the reference maximum they are relative to
         if (row / G < tpt && rtk < ntok) {
@@ -323,7 +328,8 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
                          int heads_per_group, int page_size, int page_shift, int page_run, int64_t kp, int64_t ks, int64_t kh,
                          int64_t vp, int64_t vh, int64_t vd, int max_blocks, float scale2, int window,
                          float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits, int chunk,
-                         float cap_in, float cap_out, int sink) {
+                         float cap_in, float cap_out, int sink, const float* __restrict__ sinks,
+                         const float* __restrict__ slopes) {
   __shared__ PrefillLds<HD> lds;
   // die = workgroup index mod 8. The dies form `groups` groups of `dies_per_group`, the heads as
   // many groups of `heads_per_group`; a group's (tile, head) pairs go round its dies, long tiles first.
@@ -334,7 +340,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
   const int kvh = (die / dies_per_group) * heads_per_group + item % heads_per_group;
   prefill_tile<HD, RT, PRE_WAVES, WHOLE, GENERAL>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
                        G, page_size, page_shift, page_run, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml,
-                       num_splits, chunk, blockIdx.y, cap_in, cap_out, sink);
+                       num_splits, chunk, blockIdx.y, cap_in, cap_out, sink, sinks, slopes);
 }
 
 // Keys: rows dense in head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages,
@@ -351,7 +357,7 @@ static int launch_prefill(void* out, const void* q, const void* k_cache, const v
                           int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
                           float scale, int window, int first_token, int num_tokens, int num_splits,
                           int chunk, float* part_o, float* part_ml, int page_run, bool general, float softcap, int sink,
-                          hipStream_t stream) {
+                          const float* sinks, const float* slopes, hipStream_t stream) {
   if (num_tiles <= 0) return TS_OK;
   if (general && (page_size % 32 || softcap < 0.f)) return TS_BAD_SHAPE;     // (the general variant walks whole steps only)
   const float log2e = 1.44269504088896340736f;
@@ -387,7 +393,7 @@ static int launch_prefill(void* out, const void* q, const void* k_cache, const v
   attn_prefill_mfma_kernel<HH, RR, WW, PP, GG><<<grid, WW * TS_WAVE, 0, stream>>>(                              \
       (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,             \
       seq_of_token, positions, tiles, num_tiles, nh, G, dies_per_group, heads_per_group, page_size, page_shift, page_run, kp,  \
-      ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml, num_splits, chunk, cap_in, cap_out, sink)
+      ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml, num_splits, chunk, cap_in, cap_out, sink, sinks, slopes)
 #define TS_PRE_RT(HH)                                                                                           \
   if (rt == 1) { TS_PRE_W(HH, 1, 4) } else if (rt == 2) { TS_PRE_W(HH, 2, 4) } else { TS_PRE_W(HH, 4, 4) }
 #define TS_PRE_RT8(HH)                                                                                          \
@@ -416,7 +422,8 @@ static int launch_prefill(void* out, const void* q, const void* k_cache, const v
   const int64_t skip = (int64_t)first_token * nh;     // rows of the tokens before the first listed one
   return ts_launch_attention_combine((bf16_t*)out + skip * hd, part_o + skip * num_splits * hd,
                                      part_ml + skip * num_splits * 2, positions + first_token,
-                                     num_tokens - first_token, nh, hd, num_splits, chunk, window, stream, general ? sink : 0);
+                                     num_tokens - first_token, nh, hd, num_splits, chunk, window, stream, general ? sink : 0,
+                                     general ? sinks : nullptr);
 }
 
 extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
@@ -428,11 +435,13 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
                                           int chunk, float* part_o, float* part_ml, int page_run, hipStream_t stream) {
   return launch_prefill(out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, num_tiles, tile_tokens, waves, nh,
                         nkv, hd, page_size, kp, ks, kh, vp, vh, vd, max_blocks, scale, window, first_token, num_tokens,
-                        num_splits, chunk, part_o, part_ml, page_run, false, 0.f, 0, stream);
+                        num_splits, chunk, part_o, part_ml, page_run, false, 0.f, 0, nullptr, nullptr, stream);
 }
 
 // The same with capped scores (softcap > 0: cap * tanh(score / cap)), a sink (one more in the softmax's
-// denominator) and weights carried in two bfloat16 terms; pages of a multiple of 32 keys.
+// denominator; `sinks`, float [nh], if given: exp(sinks[head]) more instead), a penalty of slopes[head] (float [nh],
+// if given) per position of distance taken off every score, and weights carried in two bfloat16 terms; pages of a
+// multiple of 32 keys.
 extern "C" int ts_paged_attention_prefill_general(void* out, const void* q, const void* k_cache, const void* v_cache,
                                                   const int32_t* block_tables, const int32_t* seq_of_token,
                                                   const int32_t* positions, const int32_t* tiles, int num_tiles,
@@ -441,8 +450,8 @@ extern "C" int ts_paged_attention_prefill_general(void* out, const void* q, cons
                                                   int max_blocks, float scale, int window, int first_token,
                                                   int num_tokens, int num_splits, int chunk, float* part_o,
                                                   float* part_ml, int page_run, float softcap, int sink,
-                                                  hipStream_t stream) {
+                                                  const float* sinks, const float* slopes, hipStream_t stream) {
   return launch_prefill(out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, num_tiles, tile_tokens, waves, nh,
                         nkv, hd, page_size, kp, ks, kh, vp, vh, vd, max_blocks, scale, window, first_token, num_tokens,
-                        num_splits, chunk, part_o, part_ml, page_run, true, softcap, sink, stream);
+                        num_splits, chunk, part_o, part_ml, page_run, true, softcap, sink || sinks, sinks, slopes, stream);
 }

@@ -227,11 +227,115 @@ moe_gemm_kernel(TO* __restrict__ out, const TX* __restrict__ x, const TX* __rest
   }
 }
 
+// bfloat16 on the matrix cores: a workgroup of four waves takes a tile's rows (TM blocks of 16) by 4 x TN x 16
+// columns, each wave TN column blocks of all the rows. Operands go from memory straight into the instruction's
+// registers: lane (r, g) holds eight consecutive k of row r of a block, 16 bytes, for the rows of x (gathered by
+// pair) as for the rows of the expert's matrix. The product is formed as y^T = W x^T, which leaves a lane four
+// consecutive columns of one row of y. With GLU a lane holds a gate sum and its up sum side by side and stores
+// the unit. K is a multiple of 32; a tile's missing rows and a matrix's missing columns are computed on
+// repeated rows and not stored.
+typedef uint32_t moe_u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
+
+static __device__ __forceinline__ moe_f32x4 moe_mfma(moe_u32x4 a, moe_u32x4 b, moe_f32x4 acc) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_bf16x8, a), __builtin_bit_cast(moe_bf16x8, b), acc, 0, 0, 0);
+}
+
+template <int TM, int TN, bool GLU, typename TO>
+__global__ void __launch_bounds__(MOE_THREADS)
+moe_gemm_mfma_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                     const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles, int src_div, int N, int K,
+                     float limit, float slope, float shift) {
+  constexpr int SETS = GLU ? 2 : 1;
+  const int tile = blockIdx.x;
+  const int rows = tiles[3 * tile + 2];
+  if (rows == 0) return;
+  const int e = tiles[3 * tile], first = tiles[3 * tile + 1];
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = (blockIdx.y * 4 + wave) * TN * 16;
+  if (n0 >= N) return;
+  const int64_t expert_rows = GLU ? 2 * (int64_t)N : N;
+  const bf16_t* we = w + (int64_t)e * expert_rows * K;
+  int pair[TM];
+  const bf16_t* xp[TM];
+  const bf16_t* wp[SETS][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    pair[i] = sorted[first + min(16 * i + r, rows - 1)];
+    xp[i] = x + (int64_t)(pair[i] / src_div) * K + 8 * g;
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = min(n0 + 16 * j + r, N - 1);
+    wp[0][j] = we + (int64_t)col * K + 8 * g;
+    if constexpr (GLU) wp[1][j] = we + (int64_t)(N + col) * K + 8 * g;
+  }
+  moe_f32x4 acc[SETS][TN][TM];
+#pragma unroll
+  for (int s = 0; s < SETS; ++s)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int i = 0; i < TM; ++i) acc[s][j][i] = (moe_f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    moe_u32x4 fx[TM], fw[SETS][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fx[i] = *(const moe_u32x4*)(xp[i] + k0);
+#pragma unroll
+    for (int s = 0; s < SETS; ++s)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fw[s][j] = *(const moe_u32x4*)(wp[s][j] + k0);
+#pragma unroll
+    for (int s = 0; s < SETS; ++s)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i) acc[s][j][i] = moe_mfma(fw[s][j], fx[i], acc[s][j][i]);
+  }
+  // lane (r, g) of block (j, i): row 16 i + r of the tile, columns n0 + 16 j + 4 g .. + 3
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    if (16 * i + r >= rows) continue;
+    TO* orow = out + (int64_t)pair[i] * N;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + 16 * j + 4 * g;
+      float y[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        if constexpr (GLU) y[c] = moe_unit(acc[0][j][i][c], acc[1][j][i][c], limit, slope, shift);
+        else y[c] = acc[0][j][i][c];
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (col + c < N) Num<TO>::st(orow + col + c, y[c]);
+    }
+  }
+}
+
 extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype, const void* w, const int32_t* sorted,
-                           const int32_t* tiles, int max_tiles, int src_div, int N, int K, int glu, float limit, float slope,
-                           float shift, hipStream_t stream) {
+                           const int32_t* tiles, int max_tiles, int tile_rows, int src_div, int N, int K, int glu, float limit,
+                           float slope, float shift, hipStream_t stream) {
   if (max_tiles <= 0) return TS_OK;
-  if (N <= 0 || K <= 0 || src_div <= 0) return TS_BAD_SHAPE;
+  if (N <= 0 || K <= 0 || src_div <= 0 || (tile_rows != 16 && tile_rows != 64)) return TS_BAD_SHAPE;
+  const bool mfma = x_dtype == 1 && K % 32 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0;
+  if (mfma) {
+    // (a wave takes 32 columns of all the tile's rows; with the gate, 32 gate and 32 up columns)
+    dim3 grid(max_tiles, (N + 127) / 128);
+    if (grid.y > 65535) return TS_BAD_SHAPE;
+#define MOE_MFMA(TM, GLU, TO) \
+    moe_gemm_mfma_kernel<TM, 2, GLU, TO><<<grid, MOE_THREADS, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w, sorted, \
+                                                                           tiles, src_div, N, K, limit, slope, shift)
+    if (glu && out_dtype == 1) { if (tile_rows == 16) MOE_MFMA(1, true, bf16_t); else MOE_MFMA(4, true, bf16_t); }
+    else if (!glu && out_dtype == 0) { if (tile_rows == 16) MOE_MFMA(1, false, float); else MOE_MFMA(4, false, float); }
+    else if (!glu && out_dtype == 1) { if (tile_rows == 16) MOE_MFMA(1, false, bf16_t); else MOE_MFMA(4, false, bf16_t); }
+    else return TS_BAD_DTYPE;
+#undef MOE_MFMA
+    return ts_check_launch();
+  }
+  if (tile_rows != MOE_BM) return TS_BAD_SHAPE;
   dim3 grid(max_tiles, (N + MOE_BN - 1) / MOE_BN);
   if (grid.y > 65535) return TS_BAD_SHAPE;
 #define MOE_LAUNCH(TX, TO) \

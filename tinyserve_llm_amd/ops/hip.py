@@ -53,9 +53,10 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, i, f,
                                       i, i, i, p],
         "ts_paged_attention_decode_general": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, i, f,
-                                              i, i, f, i, p],
+                                              i, i, f, i, p, p, p],
+        "ts_sigmoid_gate": [p, i, p, i64, i, i, p],
         "ts_paged_attention_prefill_general": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i,
-                                               i, i, p, p, i, f, i, p],
+                                               i, i, p, p, i, f, i, p, p, p],
         "ts_attention_combine": [p, p, p, p, i, i, i, i, i, i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
@@ -95,7 +96,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_conv_state_update": [p, p, i64, p, p, i, i, i, i, p],
         "ts_moe_route": [p, p, p, i, p, p, i, i, i, i, f, i, p],
         "ts_moe_group": [p, p, p, i, i, i, i, p],
-        "ts_moe_gemm": [p, i, p, i, p, p, p, i, i, i, i, i, f, f, f, p],
+        "ts_moe_gemm": [p, i, p, i, p, p, p, i, i, i, i, i, i, f, f, f, p],
         "ts_moe_combine": [p, p, p, p, i, i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
                                      i64, i64, i64, i64, p, i, p],
@@ -371,7 +372,8 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
                            seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, window: int = 0,
                            chunk: int | None = None, waves: int | None = None,
                            out: torch.Tensor | None = None, pages_per_entry: int = 1,
-                           leave_split: bool = False, softcap: float = 0.0, sink: bool = False
+                           leave_split: bool = False, softcap: float = 0.0, sink: bool = False,
+                           sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None
                            ) -> "torch.Tensor | SplitAttention":
     """Split-key attention on the matrix cores for tokens that each bring one query (bfloat16,
     values in transposed pages). Every position in `positions` must lie inside the pages its row
@@ -380,8 +382,11 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     2 to `SPLIT_ATTENTION_MAX_CHUNKS` chunks, the chunks' parts come back uncombined (a
     `SplitAttention`), for the projection that reads them. `softcap` > 0 or `sink`: the kernel's
     general variant (scores capped as softcap * tanh(score / softcap); one more in the softmax's
-    denominator; weights carried in two bfloat16 terms), which always combines."""
-    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
+    denominator; weights carried in two bfloat16 terms), which always combines; so do `sinks` (float32
+    [heads]: exp(sinks[h]) in the denominator instead of 1) and `slopes` (float32 [heads]: slopes[h] times
+    the distance between the query's position and the key's is taken off every score)."""
+    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, sinks, slopes)
+    _check_head_vectors(q.shape[1], sinks, slopes)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
     nkv = k_cache.shape[2]
@@ -406,7 +411,7 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     if splits > 1:
         part_o = torch.empty((T, nh, splits, hd), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nh, splits, 2), dtype=torch.float32, device=q.device)
-    general = softcap > 0 or sink
+    general = softcap > 0 or sink or sinks is not None or slopes is not None
     leave_split = leave_split and not general and out is None and 1 < splits <= SPLIT_ATTENTION_MAX_CHUNKS
     out = None if leave_split else _out_like(q, out)
     if general:
@@ -414,7 +419,7 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
             _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
             _ptr(seq_of_token), _ptr(positions), T, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3],
             v_cache.stride(0), v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], splits, chunk, waves,
-            float(scale), int(window), _page_run(pages_per_entry), float(softcap), int(sink), _stream()))
+            float(scale), int(window), _page_run(pages_per_entry), float(softcap), int(sink), _ptr(sinks), _ptr(slopes), _stream()))
         return out
     _run("paged_attention_decode", library().ts_paged_attention_decode(
         _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
@@ -649,7 +654,8 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             seq_of_token: torch.Tensor, positions: torch.Tensor, tiles: torch.Tensor, scale: float,
                             window: int = 0, tile_tokens: int | None = None, out: torch.Tensor | None = None,
                             num_splits: int = 1, chunk: int = 0, first_token: int = 0, waves: int = PREFILL_WAVES,
-                            pages_per_entry: int = 1, softcap: float = 0.0, sink: bool = False) -> torch.Tensor:
+                            pages_per_entry: int = 1, softcap: float = 0.0, sink: bool = False,
+                            sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of a packed step on the matrix cores (bfloat16, values in transposed pages).
     `tiles` int32 [num_tiles, 2] lists (first token, token count <= tile_tokens) per workgroup,
     every tile inside one request and inside the step (the caller built the list from the step's
@@ -660,8 +666,9 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     chunks are combined afterwards: for steps of few tokens over long contexts, which have too few
     tiles to fill the chip. The tiles must then list every token from `first_token` on.
     `pages_per_entry`: as for `paged_attention_wave`. `softcap` > 0 or `sink`: the kernel's general
-    variant, as for `paged_attention_decode` (cache pages of a multiple of 32 keys)."""
-    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles)
+    variant, as for `paged_attention_decode` (cache pages of a multiple of 32 keys); `sinks`, `slopes`: as there."""
+    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, sinks, slopes)
+    _check_head_vectors(q.shape[1], sinks, slopes)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
     nkv = k_cache.shape[2]
@@ -692,9 +699,10 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
             _ptr(tiles), tiles.shape[0], tile_tokens, waves, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
             v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], float(scale), int(window), first_token, T,
             num_splits, chunk, _ptr(part_o), _ptr(part_ml), _page_run(pages_per_entry))
-    if softcap > 0 or sink:
+    if softcap > 0 or sink or sinks is not None or slopes is not None:
         _need(k_cache.shape[1] % 32 == 0, "the general variant takes cache pages of a multiple of 32 keys")
-        _run("paged_attention_prefill_general", library().ts_paged_attention_prefill_general(*args, float(softcap), int(sink), _stream()))
+        _run("paged_attention_prefill_general", library().ts_paged_attention_prefill_general(
+            *args, float(softcap), int(sink), _ptr(sinks), _ptr(slopes), _stream()))
     else:
         _run("paged_attention_prefill", library().ts_paged_attention_prefill(*args, _stream()))
     return out
@@ -702,15 +710,21 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int,
                     scale: float, window: int = 0, leave_split: bool = False, softcap: float = 0.0,
-                    sink: bool = False) -> "torch.Tensor | SplitAttention":
+                    sink: bool = False, sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None,
+                    gate: torch.Tensor | None = None) -> "torch.Tensor | SplitAttention":
     """Attention of a packed step over the cache; picks the kernel for the storage type and shape.
     float32 always takes the one-wave-per-row kernel, whose sums do not depend on the batch;
     bfloat16 takes the matrix-core kernels where they serve the shape. `leave_split`: a step of single
     tokens whose keys are walked in chunks may come back as a `SplitAttention` (see `paged_attention_decode`).
     `softcap` > 0 (scores capped as softcap * tanh(score / softcap)) or `sink` (one more in the softmax's
     denominator) choose the kernels' general variants; those, and value rows of a size of their own, fall
-    back to `paged_attention_general`, which is 32-bit throughout."""
-    general = softcap > 0 or sink
+    back to `paged_attention_general`, which is 32-bit throughout. `sinks` / `slopes` (float32 [heads]): learned
+    sinks (exp(sinks[h]) in the denominator) and a penalty of slopes[h] per position of distance on every score,
+    by the general variants likewise. `gate` (float32 [tokens, heads * value_dim], rows may lie apart): the
+    output is multiplied element by element by sigmoid(gate), by the 32-bit kernel on its way out or by a
+    kernel of its own behind the matrix-core kernels."""
+    general = softcap > 0 or sink or sinks is not None or slopes is not None or gate is not None
+    extra = dict(softcap=softcap, sink=sink, sinks=sinks, slopes=slopes)
     tables = ctx.block_tables[space]
     # (the tables count in pages of ctx.page_size tokens; the pools may be cut into shorter ones)
     table_page = getattr(ctx, "page_size", 0) or k_cache.shape[1]
@@ -721,8 +735,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         capacity = tables.shape[1] * table_page
         decode_ok = -(-capacity // 1024) <= MAX_DECODE_SPLITS and q.shape[0] <= MAX_DECODE_TOKENS
         if ctx.max_query_len == 1 and decode_ok:
-            return paged_attention_decode(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window,
-                                          pages_per_entry=per_entry, leave_split=leave_split, softcap=softcap, sink=sink)
+            return _gated(paged_attention_decode(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window,
+                                                 pages_per_entry=per_entry, leave_split=leave_split and gate is None, **extra), gate)
         # the one-token requests that lead the step go to the split-key kernel, the rest to the tiles
         cu = ctx.host_cu_seqlens
         lead = 0
@@ -741,14 +755,14 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         out = torch.empty_like(q)
         if lead:
             paged_attention_decode(q[:lead], k_cache, v_cache, tables, ctx.seq_of_token[:lead], ctx.positions[:lead],
-                                   scale, window, out=out[:lead], pages_per_entry=per_entry, softcap=softcap, sink=sink)
+                                   scale, window, out=out[:lead], pages_per_entry=per_entry, **extra)
         splits, chunk = prefill_splits(tiles.shape[0] * nkv, max(ctx.host_context_lens[lead:], default=0))
-        return paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale,
-                                       window, tile_tokens=tile_tokens, out=out, num_splits=splits, chunk=chunk,
-                                       first_token=cu[lead], waves=waves, pages_per_entry=per_entry, softcap=softcap, sink=sink)
+        return _gated(paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale,
+                                              window, tile_tokens=tile_tokens, out=out, num_splits=splits, chunk=chunk,
+                                              first_token=cu[lead], waves=waves, pages_per_entry=per_entry, **extra), gate)
     if general or k_cache.shape[3] != v_cache.shape[3]:
         return paged_attention_general(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, softcap=softcap,
-                                       sink=sink, window=window, pages_per_entry=per_entry)
+                                       sink=sink, window=window, pages_per_entry=per_entry, sinks=sinks, slopes=slopes, gate=gate)
     return paged_attention_wave(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window,
                                 pages_per_entry=per_entry)
 
@@ -1740,12 +1754,18 @@ def qkv_finish(qkv: torch.Tensor, freqs: torch.Tensor | None, positions: torch.T
 
 def paged_attention_general(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                             seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, *, softcap: float = 0.0,
-                            sink: bool = False, window: int = 0, pages_per_entry: int = 1) -> torch.Tensor:
+                            sink: bool = False, window: int = 0, pages_per_entry: int = 1, sinks: torch.Tensor | None = None,
+                            slopes: torch.Tensor | None = None, gate: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of each token (at its position, causal, optionally windowed) over its request's
     pages, in 32-bit: score = q.k * scale, capped as softcap * tanh(score / softcap) if softcap > 0;
     with `sink` the softmax has one more in its denominator (a key of score 0 without a value).
-    Value rows may differ in size from key rows: out [tokens, heads, value_dim]."""
-    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions)
+    Value rows may differ in size from key rows: out [tokens, heads, value_dim]. `sinks` (float32 [heads]):
+    the sink's score is sinks[h] instead of 0; `slopes` (float32 [heads]): slopes[h] * (query position - key
+    position) is taken off every score; `gate` (float32 [tokens, heads * value_dim], a view whose rows may lie
+    apart): the output row is multiplied by sigmoid(gate) element by element."""
+    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, sinks, slopes, gate)
+    _check_head_vectors(q.shape[1], sinks, slopes)
+    gate_stride = _check_gate(gate, q.shape[0], q.shape[1] * v_cache.shape[3])
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
     nkv, vd = k_cache.shape[2], v_cache.shape[3]
@@ -1759,46 +1779,39 @@ def paged_attention_general(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     _run("paged_attention_general", library().ts_paged_attention_general(
         _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_of_token), _ptr(positions),
         T, nh, nkv, hd, vd, k_cache.shape[1], *k_cache.stride()[:3], *v_cache.stride(), block_tables.shape[1],
-        float(scale), float(softcap), int(sink), int(window), _code(q.dtype), _page_run(pages_per_entry), None, None, None, 0,
-        _stream()))
-    return out
-
-
-def paged_attention_sloped(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int, scale: float, *,
-                           window: int = 0, sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None,
-                           gate: torch.Tensor | None = None) -> torch.Tensor:
-    """Attention of a packed step over the cache in 32-bit, with what `paged_attention` has no argument for:
-    `slopes` (float32 [heads]): slopes[h] * (query position - key position) is taken off every score;
-    `sinks` (float32 [heads]): the softmax's denominator also holds exp(sinks[h]) (a key without a value);
-    `gate` (float32 [tokens, >= heads * value_dim], a view whose rows may lie apart): the output row is
-    multiplied by sigmoid(gate) element by element. out [tokens, heads, value_dim] in q's type."""
-    _gpu(q, k_cache, v_cache, sinks, slopes, gate)
-    _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
-    T, nh, hd = q.shape
-    nkv, vd = k_cache.shape[2], v_cache.shape[3]
-    _check_cache_pair(k_cache, v_cache, q.dtype, nkv, hd, vd)
-    _need(nh % nkv == 0, lambda: f"{nh} heads do not divide into {nkv} key/value heads")
-    tables, seq_of_token, positions = ctx.block_tables[space], ctx.seq_of_token, ctx.positions
-    table_page = getattr(ctx, "page_size", 0) or k_cache.shape[1]
-    _need(table_page % k_cache.shape[1] == 0, lambda: f"block tables in pages of {table_page} over a cache in pages of {k_cache.shape[1]}")
-    _need(tables.dtype == torch.int32 and tables.dim() == 2 and tables.is_contiguous(),
-          "block_tables must be contiguous int32 [requests, pages]")
-    for name, t in (("seq_of_token", seq_of_token), ("positions", positions)):
-        _need(t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous(), lambda: f"{name} must be int32 [tokens]")
-    for name, t in (("sinks", sinks), ("slopes", slopes)):
-        _need(t is None or (t.dtype == torch.float32 and t.shape == (nh,) and t.is_contiguous()), lambda: f"{name} must be float32 [heads]")
-    gate_stride = 0
-    if gate is not None:
-        _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape == (T, nh * vd) and gate.stride(1) == 1
-              and gate.stride(0) >= nh * vd, "the gate must be float32 [tokens, heads * value_dim] with contiguous rows")
-        gate_stride = gate.stride(0)
-    out = torch.empty((T, nh, vd), dtype=q.dtype, device=q.device)
-    _run("paged_attention_general", library().ts_paged_attention_general(
-        _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(tables), _ptr(seq_of_token), _ptr(positions),
-        T, nh, nkv, hd, vd, k_cache.shape[1], *k_cache.stride()[:3], *v_cache.stride(), tables.shape[1],
-        float(scale), 0.0, 0, int(window), _code(q.dtype), _page_run(table_page // k_cache.shape[1]), _ptr(sinks), _ptr(slopes),
+        float(scale), float(softcap), int(sink), int(window), _code(q.dtype), _page_run(pages_per_entry), _ptr(sinks), _ptr(slopes),
         _ptr(gate), gate_stride, _stream()))
     return out
+
+
+def _check_head_vectors(heads: int, *vectors: torch.Tensor | None) -> None:
+    for t in vectors:
+        _need(t is None or (t.dtype == torch.float32 and t.shape == (heads,) and t.is_contiguous()), "a number per head: float32 [heads]")
+
+
+def _check_gate(gate: torch.Tensor | None, tokens: int, width: int) -> int:
+    """The stride between a gate's rows (0 if there is none)."""
+    if gate is None:
+        return 0
+    _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape == (tokens, width) and gate.stride(1) == 1
+          and gate.stride(0) >= width, "the gate must be float32 [tokens, heads * value_dim] with contiguous rows")
+    return gate.stride(0)
+
+
+def sigmoid_gate_(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """x *= sigmoid(gate) in place, element by element (x [tokens, ...] contiguous, float32 or bfloat16; gate
+    float32 [tokens, width] with contiguous rows that may lie apart)."""
+    _gpu(x, gate)
+    _need(x.is_contiguous(), "the rows to gate must be contiguous")
+    tokens = x.shape[0]
+    width = x.numel() // max(tokens, 1)
+    stride = _check_gate(gate, tokens, width)
+    _run("sigmoid_gate", library().ts_sigmoid_gate(_ptr(x), _code(x.dtype), _ptr(gate), stride, tokens, width, _stream()))
+    return x
+
+
+def _gated(out, gate: torch.Tensor | None):
+    return out if gate is None else sigmoid_gate_(out, gate)
 
 
 # ---- the dynamic-tanh norm ----
@@ -1950,7 +1963,8 @@ def conv_state_update(state: torch.Tensor, proj: torch.Tensor, ctx) -> None:
 
 # ---- a mixture of experts ----
 
-MOE_TILE_ROWS = 16
+MOE_TILE_ROWS = 16        # rows of a tile of the experts' products,
+MOE_WIDE_TILE_ROWS = 64   # or, in bfloat16, where the experts have this many rows each on average
 MOE_MAX_EXPERTS = 1024
 MOE_MAX_TOP = 32
 
@@ -1978,20 +1992,30 @@ class ExpertTiles:
     """A step's (token, choice) pairs grouped by expert: `sorted` int32 [pairs] (pair indices, an expert's
     side by side), `tiles` int32 [max_tiles, 3] = (expert, first index into `sorted`, rows; rows 0: unused)."""
 
-    def __init__(self, sorted_pairs: torch.Tensor, tiles: torch.Tensor, top: int, experts: int) -> None:
-        self.sorted, self.tiles, self.top, self.experts = sorted_pairs, tiles, top, experts
+    def __init__(self, sorted_pairs: torch.Tensor, tiles: torch.Tensor, top: int, experts: int, tile_rows: int) -> None:
+        self.sorted, self.tiles, self.top, self.experts, self.tile_rows = sorted_pairs, tiles, top, experts, tile_rows
 
 
-def moe_group(ids: torch.Tensor, experts: int) -> ExpertTiles:
+def moe_tile_rows(pairs: int, experts: int, dtype: torch.dtype, k_sizes: "tuple[int, ...]" = ()) -> int:
+    """Rows of a tile for a step of `pairs` (token, expert) pairs: the wide tile where the matrix-core kernel
+    runs (bfloat16, reductions that are multiples of 32) and an expert has that many rows on average, so
+    that an expert's matrix is read once per 64 rows and not once per 16."""
+    wide = dtype == torch.bfloat16 and all(k % 32 == 0 for k in k_sizes) and pairs >= MOE_WIDE_TILE_ROWS * experts
+    return MOE_WIDE_TILE_ROWS if wide else MOE_TILE_ROWS
+
+
+def moe_group(ids: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS) -> ExpertTiles:
+    """Groups the step's pairs by expert and cuts the groups into tiles of up to `tile_rows` rows."""
     _gpu(ids)
+    _need(tile_rows in (MOE_TILE_ROWS, MOE_WIDE_TILE_ROWS), "tiles of 16 or 64 rows")
     _need(ids.dtype == torch.int32 and ids.dim() == 2 and ids.is_contiguous(), "the chosen experts must be contiguous int32 [tokens, top]")
     _need(0 < experts <= MOE_MAX_EXPERTS, lambda: f"up to {MOE_MAX_EXPERTS} experts")
     P = ids.numel()
-    max_tiles = P // MOE_TILE_ROWS + min(experts, P)
+    max_tiles = P // tile_rows + min(experts, P)
     sorted_pairs = torch.empty((P,), dtype=torch.int32, device=ids.device)
     tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=ids.device)
-    _run("moe_group", library().ts_moe_group(_ptr(ids), _ptr(sorted_pairs), _ptr(tiles), P, experts, MOE_TILE_ROWS, max_tiles, _stream()))
-    return ExpertTiles(sorted_pairs, tiles, ids.shape[1], experts)
+    _run("moe_group", library().ts_moe_group(_ptr(ids), _ptr(sorted_pairs), _ptr(tiles), P, experts, tile_rows, max_tiles, _stream()))
+    return ExpertTiles(sorted_pairs, tiles, ids.shape[1], experts, tile_rows)
 
 
 def moe_gemm(x: torch.Tensor, weights: torch.Tensor, grouped: ExpertTiles, out_dtype: torch.dtype, *, per_token: bool,
@@ -2011,8 +2035,10 @@ def moe_gemm(x: torch.Tensor, weights: torch.Tensor, grouped: ExpertTiles, out_d
         n //= 2
     out = torch.empty((P, n), dtype=out_dtype, device=x.device)
     limit, slope, shift = glu if glu is not None else (0.0, 0.0, 0.0)
+    _need(grouped.tile_rows == MOE_TILE_ROWS or (x.dtype == torch.bfloat16 and x.shape[1] % 32 == 0),
+          "wide tiles are the matrix-core kernel's: bfloat16, a reduction that is a multiple of 32")
     _run("moe_gemm", library().ts_moe_gemm(_ptr(out), _code(out_dtype), _ptr(x), _code(x.dtype), _ptr(weights), _ptr(grouped.sorted),
-                                           _ptr(grouped.tiles), grouped.tiles.shape[0], grouped.top if per_token else 1, n, x.shape[1],
+                                           _ptr(grouped.tiles), grouped.tiles.shape[0], grouped.tile_rows, grouped.top if per_token else 1, n, x.shape[1],
                                            int(glu is not None), float(limit), float(slope), float(shift), _stream()))
     return out
 

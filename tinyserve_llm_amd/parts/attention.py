@@ -291,7 +291,6 @@ class ConvAttention(Mixer):
                             eps=self.qk_norm_eps or 0.0, temp_coef=self.q_temp_coef, temp_every=self.q_temp_every)
         if self.conv_taps > 1:
             hip.conv_state_update(mem.state, proj, ctx)
-        o = hip.paged_attention_sloped(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, window=self.window,
-                                       sinks=self.sink, slopes=self.slopes,
-                                       gate=proj[:, self.channels:] if self.has_gate else None)
+        o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window, sinks=self.sink,
+                                slopes=self.slopes, gate=proj[:, self.channels:] if self.has_gate else None)
         return linear(o.view(ctx.num_tokens, self.out_size), self.o, out_dtype=torch.float32, packed=self.o_packed)

@@ -64,7 +64,8 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         experts, weights = hip.moe_route(x, self.router, self.correction, self.top, self.router_scale, self.normalize)
-        grouped = hip.moe_group(experts, self.num_experts)
+        tile_rows = hip.moe_tile_rows(experts.numel(), self.num_experts, x.dtype, (self.hidden_size, self.intermediate_size))
+        grouped = hip.moe_group(experts, self.num_experts, tile_rows)
         unit = hip.moe_gemm(x, self.gate_up, grouped, x.dtype, per_token=True, glu=(self.limit, self.slope, self.up_shift))
         rows = hip.moe_gemm(unit, self.down, grouped, torch.float32, per_token=False)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
