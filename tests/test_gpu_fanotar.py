@@ -150,7 +150,7 @@ def test_convolution_norms_multiplier_cache_and_state(in_dtype, dtype, shape):
     H, G, D, V, taps, (coef, every) = shape
     C = (H + G) * D + G * V
     extra = 24                                              # (columns after the channels: a gate's)
-    lengths, page = [37, 9, 21], 8
+    lengths, page = [300, 9, 21], 8                        # (one step of more than 256 tokens: its values leave in tiles)
     conv = (torch.randn(C, taps) * 0.4 + 1.0 / taps).to(DEV)
     qn, kn = (1 + 0.2 * torch.randn(D)).to(DEV), (1 + 0.2 * torch.randn(D)).to(DEV)
     proj = [rounded(torch.randn(n, C + extra), in_dtype) for n in lengths]
@@ -173,7 +173,7 @@ def test_convolution_norms_multiplier_cache_and_state(in_dtype, dtype, shape):
         if G:
             want_k.append(plain.unit_rms(y[:, H * D:(H + G) * D].view(n, G, D), eps) * kn.cpu().to(F64))
             want_v.append(y[:, (H + G) * D:].view(n, G, V))
-    cuts = [[1, 2, 1, 5, 2, 26], [2, 1, 1, 1, 4], [7, 1, 13]]
+    cuts = [[1, 2, 1, 5, 2, 289], [2, 1, 1, 1, 4], [7, 1, 13]]
     cursors, got_q = [0, 0, 0], [[], [], []]
     for step in range(max(len(c) for c in cuts)):
         live = [i for i in range(3) if step < len(cuts[i])]
@@ -296,7 +296,7 @@ def test_the_sink_weighs_most_on_the_first_tokens():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("sizes", [(6, 3, 80, 40, 23), (4, 1, 48, 20, 1), (5, 5, 99, 17, 9), (12, 2, 64, 24, 70), (8, 2, 512, 128, 40),
-                                   (4, 2, 64, 32, 170), (3, 1, 96, 160, 400)])
+                                   (4, 2, 64, 32, 170), (3, 1, 96, 160, 300), (3, 2, 128, 192, 300), (2, 1, 192, 64, 513)])
 def test_router_grouping_and_experts(dtype, sizes):
     h = hip()
     E, top, W, F, n = sizes
@@ -321,7 +321,9 @@ def test_router_grouping_and_experts(dtype, sizes):
     down, d64 = rounded(torch.randn(E, W, F) * F ** -0.5, dtype)
     # (the last two cases give an expert enough rows for the wide tiles of the matrix-core kernel in bfloat16)
     tile_rows = h.moe_tile_rows(n * top, E, dtype, (W, F))
-    assert tile_rows == (64 if dtype == torch.bfloat16 and n >= 170 else 16)
+    # (the last cases give an expert enough rows for the tiles of 64 and of 128 rows in bfloat16)
+    wide = 16 if dtype != torch.bfloat16 or n < 170 else 128 if n * top >= 128 * E and W % 64 == 0 and F % 64 == 0 else 64
+    assert tile_rows == wide
     grouped = h.moe_group(ids, E, tile_rows)
     tiles = grouped.tiles.cpu()
     assert sorted(grouped.sorted.cpu().tolist()) == list(range(n * top))

@@ -19,44 +19,84 @@
 #define MOE_MAX_EXPERTS 1024
 #define MOE_MAX_TOP 32
 
+#define MOE_ROUTE_CHUNK 2048      // elements of a token's row that lie in LDS at a time
+#define MOE_ROUTE_THREADS 1024    // sixteen waves: an expert each at a time, so that a step of few tokens has all its loads in flight at once
+
 template <typename TX>
-__global__ void __launch_bounds__(MOE_THREADS)
+__global__ void __launch_bounds__(MOE_ROUTE_THREADS)
 moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const TX* __restrict__ x,
                  const float* __restrict__ router, const float* __restrict__ correction, int num_tokens, int K, int E, int top,
                  float scale, int normalize) {
   extern __shared__ float lds[];
-  float* s_s = lds;                                       // [MOE_ROUTE_TOKENS][E] scores
+  float* s_s = lds;                                       // [MOE_ROUTE_TOKENS][E] logits, then scores
   float* c_s = lds + MOE_ROUTE_TOKENS * E;                // [MOE_ROUTE_TOKENS][E] choice scores
+  float* x_s = c_s + MOE_ROUTE_TOKENS * E;                // [MOE_ROUTE_TOKENS][MOE_ROUTE_CHUNK] the tokens' rows, 32-bit
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
   const int t0 = blockIdx.x * MOE_ROUTE_TOKENS;
   const int nt = min(MOE_ROUTE_TOKENS, num_tokens - t0);
-  for (int e = wave; e < E; e += MOE_THREADS / TS_WAVE) {
-    float acc[MOE_ROUTE_TOKENS];
-#pragma unroll
-    for (int r = 0; r < MOE_ROUTE_TOKENS; ++r) acc[r] = 0.f;
-    const float* wr = router + (int64_t)e * K;
-    for (int k = lane; k < K; k += TS_WAVE) {
-      const float w = wr[k];
-#pragma unroll
-      for (int r = 0; r < MOE_ROUTE_TOKENS; ++r)
-        if (r < nt) acc[r] = fmaf(w, Num<TX>::ld(x + (int64_t)(t0 + r) * K + k), acc[r]);
+  for (int i = threadIdx.x; i < MOE_ROUTE_TOKENS * E; i += MOE_ROUTE_THREADS) s_s[i] = 0.f;
+  const bool by4 = K % 4 == 0 && ((uintptr_t)router & 15) == 0;     // (rows of the router in 16-byte pieces)
+  // a stretch of the rows into LDS, then every wave takes experts in turn: a lane reads the router's row side by
+  // side with its neighbours, all of a stretch's pieces asked for before the first is used
+  for (int k0 = 0; k0 < K; k0 += MOE_ROUTE_CHUNK) {
+    const int kn = min(MOE_ROUTE_CHUNK, K - k0);
+    __syncthreads();
+#pragma unroll 8
+    for (int i = threadIdx.x; i < MOE_ROUTE_TOKENS * kn; i += MOE_ROUTE_THREADS) {
+      const int r = i / kn, k = i - r * kn;
+      x_s[r * MOE_ROUTE_CHUNK + k] = r < nt ? Num<TX>::ld(x + (int64_t)(t0 + r) * K + k0 + k) : 0.f;
     }
+    __syncthreads();
+    for (int e = wave; e < E; e += MOE_ROUTE_THREADS / TS_WAVE) {
+      float acc[MOE_ROUTE_TOKENS];
 #pragma unroll
-    for (int r = 0; r < MOE_ROUTE_TOKENS; ++r) {
-      const float z = wave_sum(acc[r]);
-      if (lane == 0) {
-        const float s = 1.0f / (1.0f + expf(-z));
-        s_s[r * E + e] = s;
-        c_s[r * E + e] = s + (correction ? correction[e] : 0.f);
+      for (int r = 0; r < MOE_ROUTE_TOKENS; ++r) acc[r] = 0.f;
+      const float* wr = router + (int64_t)e * K + k0;
+      if (by4) {
+        constexpr int PIECES = MOE_ROUTE_CHUNK / (4 * TS_WAVE);
+        float4 w[PIECES];
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+          const int k = 4 * (lane + TS_WAVE * i);
+          w[i] = k < kn ? *(const float4*)(wr + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+          const int k = 4 * (lane + TS_WAVE * i);
+          if (k >= kn) continue;
+#pragma unroll
+          for (int r = 0; r < MOE_ROUTE_TOKENS; ++r) {
+            const float4 xv = *(const float4*)(x_s + r * MOE_ROUTE_CHUNK + k);
+            acc[r] = fmaf(w[i].x, xv.x, fmaf(w[i].y, xv.y, fmaf(w[i].z, xv.z, fmaf(w[i].w, xv.w, acc[r]))));
+          }
+        }
+      } else {
+#pragma unroll 8
+        for (int k = lane; k < kn; k += TS_WAVE) {
+          const float w = wr[k];
+#pragma unroll
+          for (int r = 0; r < MOE_ROUTE_TOKENS; ++r) acc[r] = fmaf(w, x_s[r * MOE_ROUTE_CHUNK + k], acc[r]);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < MOE_ROUTE_TOKENS; ++r) {
+        const float z = wave_sum(acc[r]);
+        if (lane == 0) s_s[r * E + e] += z;                // (an expert is one wave's: no other adds to it)
       }
     }
   }
   __syncthreads();
+  for (int i = threadIdx.x; i < MOE_ROUTE_TOKENS * E; i += MOE_ROUTE_THREADS) {
+    const float sc = 1.0f / (1.0f + expf(-s_s[i]));
+    s_s[i] = sc;
+    c_s[i] = sc + (correction ? correction[i % E] : 0.f);
+  }
+  __syncthreads();
   if (wave >= nt) return;                                 // a wave per token from here on
   const int r = wave, t = t0 + wave;
-  float total = 0.f;
-  float picked[MOE_MAX_TOP];
-  int chosen[MOE_MAX_TOP];
+  // lane j keeps the j-th choice (top <= 32 lanes of the 64)
+  float my_pick = 0.f;
+  int my_choice = 0;
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
     int at = 0x7fffffff;
@@ -71,19 +111,17 @@ moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const
       if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
     }
     if (at >= E) at = j;                                  // (scores that are no numbers: still valid indices)
-    chosen[j] = at;
-    picked[j] = s_s[r * E + at];
-    total += picked[j];
+    if (lane == j) { my_choice = at; my_pick = s_s[r * E + at]; }
     wave_sync();
     if (lane == 0) c_s[r * E + at] = -INFINITY;
     wave_sync();
   }
+  const float total = wave_sum(my_pick);                  // (the lanes beyond `top` hold 0)
   const float mult = (normalize ? 1.0f / (total + 1e-20f) : 1.0f) * scale;
-  if (lane == 0)
-    for (int j = 0; j < top; ++j) {
-      ids_out[(int64_t)t * top + j] = chosen[j];
-      w_out[(int64_t)t * top + j] = picked[j] * mult;
-    }
+  if (lane < top) {
+    ids_out[(int64_t)t * top + lane] = my_choice;
+    w_out[(int64_t)t * top + lane] = my_pick * mult;
+  }
 }
 
 extern "C" int ts_moe_route(int32_t* ids_out, float* w_out, const void* x, int x_dtype, const float* router,
@@ -92,13 +130,13 @@ extern "C" int ts_moe_route(int32_t* ids_out, float* w_out, const void* x, int x
   if (num_tokens <= 0) return TS_OK;
   if (K <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > MOE_MAX_TOP || top > E) return TS_BAD_SHAPE;
   const unsigned blocks = (num_tokens + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS;
-  const size_t lds = (size_t)2 * MOE_ROUTE_TOKENS * E * sizeof(float);
+  const size_t lds = (size_t)MOE_ROUTE_TOKENS * (2 * E + MOE_ROUTE_CHUNK) * sizeof(float);
   if (x_dtype == 0)
-    moe_route_kernel<float><<<blocks, MOE_THREADS, lds, stream>>>(ids_out, w_out, (const float*)x, router, correction, num_tokens,
-                                                                  K, E, top, scale, normalize);
+    moe_route_kernel<float><<<blocks, MOE_ROUTE_THREADS, lds, stream>>>(ids_out, w_out, (const float*)x, router, correction,
+                                                                        num_tokens, K, E, top, scale, normalize);
   else if (x_dtype == 1)
-    moe_route_kernel<bf16_t><<<blocks, MOE_THREADS, lds, stream>>>(ids_out, w_out, (const bf16_t*)x, router, correction,
-                                                                   num_tokens, K, E, top, scale, normalize);
+    moe_route_kernel<bf16_t><<<blocks, MOE_ROUTE_THREADS, lds, stream>>>(ids_out, w_out, (const bf16_t*)x, router, correction,
+                                                                         num_tokens, K, E, top, scale, normalize);
   else return TS_BAD_DTYPE;
   return ts_check_launch();
 }
@@ -315,12 +353,161 @@ moe_gemm_mfma_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const b
   }
 }
 
+// Tiles of 128 rows, for steps that give an expert hundreds of rows: both operands go through LDS in the order the
+// matrix instruction wants them (lane (r, g) of fragment f: row 16 (f / 2) + r, elements 32 (f % 2) + 8 g .. + 7),
+// 64 of K at a time, two k-steps in flight (one in an LDS buffer being multiplied, the next in registers on its way
+// into the other buffer), as in the engine's tiled product for plain matrices; here the rows of x are gathered by
+// pair, the matrix is the tile's expert's, and the rows of y go to their pairs' places. A workgroup of WM x WN
+// waves takes 128 rows by 128 columns (with GLU: 64 gate and 64 up columns, whose sums meet in one lane). K is a
+// multiple of 64.
+template <int WM, int WN, bool GLU, typename TO>
+__global__ void __launch_bounds__(WM * WN * TS_WAVE)
+moe_gemm_lds_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                    const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles, int src_div, int N, int K,
+                    float limit, float slope, float shift) {
+  constexpr int BM = 128, BN = 128;
+  constexpr int THREADS = WM * WN * TS_WAVE;
+  constexpr int FX = BM / 16 * 2, FW = BN / 16 * 2;       // fragments (a kilobyte each) of a k-step of 64
+  constexpr int TM = BM / WM / 16, TN = BN / WN / 16;     // 16 x 16 blocks of a wave
+  constexpr int LX = FX * 64 / THREADS, LW = FW * 64 / THREADS;
+  static_assert(!GLU || WN == 1, "a gate sum and its up sum must meet in one wave");
+  __shared__ moe_u32x4 lds[2][(FX + FW) * 64];
+  const int tile = blockIdx.x;
+  const int rows = tiles[3 * tile + 2];
+  if (rows == 0) return;
+  const int e = tiles[3 * tile], first = tiles[3 * tile + 1];
+  // (with GLU a workgroup's 128 columns of the product are 64 columns of y)
+  const int n0 = blockIdx.y * (GLU ? BN / 2 : BN);
+  const int t = threadIdx.x, lane = t % TS_WAVE, r = lane % 16, g = lane / 16;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TS_WAVE), wm = wave % WM, wn = wave / WM;
+  const bf16_t* we = w + (int64_t)e * (GLU ? 2 : 1) * N * K;
+  const bf16_t* xp[LX];
+  const bf16_t* wp[LW];
+#pragma unroll
+  for (int i = 0; i < LX; ++i) {
+    const int f = (t + THREADS * i) / 64;
+    const int pair = sorted[first + min((f / 2) * 16 + r, rows - 1)];
+    xp[i] = x + (int64_t)(pair / src_div) * K + (f % 2) * 32 + 8 * g;
+  }
+#pragma unroll
+  for (int i = 0; i < LW; ++i) {
+    const int f = (t + THREADS * i) / 64;
+    int col = (f / 2) * 16 + r;
+    if (GLU) col = min(n0 + col % (BN / 2), N - 1) + (col >= BN / 2 ? N : 0);
+    else col = min(n0 + col, N - 1);
+    wp[i] = we + (int64_t)col * K + (f % 2) * 32 + 8 * g;
+  }
+  moe_u32x4 sx0[LX], sw0[LW], sx1[LX], sw1[LW];
+  moe_f32x4 acc[TN][TM];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int i = 0; i < TM; ++i) acc[j][i] = (moe_f32x4){0.f, 0.f, 0.f, 0.f};
+#define MOE_FETCH(S, k0)                                                                                  \
+  do {                                                                                                    \
+    _Pragma("unroll") for (int i = 0; i < LX; ++i) sx##S[i] = *(const moe_u32x4*)(xp[i] + (k0));          \
+    _Pragma("unroll") for (int i = 0; i < LW; ++i) sw##S[i] = *(const moe_u32x4*)(wp[i] + (k0));          \
+  } while (0)
+#define MOE_STASH(S)                                                                                      \
+  do {                                                                                                    \
+    _Pragma("unroll") for (int i = 0; i < LX; ++i) lds[S][t + THREADS * i] = sx##S[i];                    \
+    _Pragma("unroll") for (int i = 0; i < LW; ++i) lds[S][FX * 64 + t + THREADS * i] = sw##S[i];          \
+  } while (0)
+#define MOE_MULTIPLY(S)                                                                                   \
+  _Pragma("unroll") for (int h = 0; h < 2; ++h) {                                                         \
+    moe_u32x4 fx[TM], fw[TN];                                                                             \
+    _Pragma("unroll") for (int i = 0; i < TM; ++i) fx[i] = lds[S][((wm * TM + i) * 2 + h) * 64 + lane];   \
+    _Pragma("unroll") for (int j = 0; j < TN; ++j) fw[j] = lds[S][FX * 64 + ((wn * TN + j) * 2 + h) * 64 + lane]; \
+    _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                        \
+      _Pragma("unroll") for (int i = 0; i < TM; ++i) acc[j][i] = moe_mfma(fw[j], fx[i], acc[j][i]);       \
+  }
+  const int steps = K / 64;
+  MOE_FETCH(0, 0);
+  if (steps == 1) {
+    MOE_STASH(0);
+    __syncthreads();
+    MOE_MULTIPLY(0)
+  } else {
+    MOE_FETCH(1, 64);
+    MOE_STASH(0);
+    __syncthreads();
+    int s = 0;
+    for (; s + 3 < steps; s += 2) {
+      MOE_FETCH(0, 64 * (s + 2));
+      MOE_MULTIPLY(0)
+      MOE_STASH(1);
+      __syncthreads();
+      MOE_FETCH(1, 64 * (s + 3));
+      MOE_MULTIPLY(1)
+      MOE_STASH(0);
+      __syncthreads();
+    }
+    // two or three steps are left: step s in buffer 0, step s + 1 in register set 1
+    if (steps - s == 3) {
+      MOE_FETCH(0, 64 * (s + 2));
+      MOE_MULTIPLY(0)
+      MOE_STASH(1);
+      __syncthreads();
+      MOE_MULTIPLY(1)
+      MOE_STASH(0);
+      __syncthreads();
+      MOE_MULTIPLY(0)
+    } else {
+      MOE_MULTIPLY(0)
+      MOE_STASH(1);
+      __syncthreads();
+      MOE_MULTIPLY(1)
+    }
+  }
+#undef MOE_FETCH
+#undef MOE_STASH
+#undef MOE_MULTIPLY
+  // lane (r, g) of block (j, i): row 16 (wm TM + i) + r of the tile, columns .. + 4 g .. + 3
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = (wm * TM + i) * 16 + r;
+    if (m >= rows) continue;
+    TO* orow = out + (int64_t)sorted[first + m] * N;
+    if constexpr (GLU) {
+#pragma unroll
+      for (int j = 0; j < TN / 2; ++j) {
+        const int n = n0 + j * 16 + 4 * g;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (n + c < N) Num<TO>::st(orow + n + c, moe_unit(acc[j][i][c], acc[j + TN / 2][i][c], limit, slope, shift));
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int n = n0 + (wn * TN + j) * 16 + 4 * g;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (n + c < N) Num<TO>::st(orow + n + c, acc[j][i][c]);
+      }
+    }
+  }
+}
+
 extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype, const void* w, const int32_t* sorted,
                            const int32_t* tiles, int max_tiles, int tile_rows, int src_div, int N, int K, int glu, float limit,
                            float slope, float shift, hipStream_t stream) {
   if (max_tiles <= 0) return TS_OK;
-  if (N <= 0 || K <= 0 || src_div <= 0 || (tile_rows != 16 && tile_rows != 64)) return TS_BAD_SHAPE;
+  if (N <= 0 || K <= 0 || src_div <= 0 || (tile_rows != 16 && tile_rows != 64 && tile_rows != 128)) return TS_BAD_SHAPE;
   const bool mfma = x_dtype == 1 && K % 32 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0;
+  if (tile_rows == 128) {
+    if (!mfma || K % 64) return TS_BAD_SHAPE;
+    dim3 grid(max_tiles, glu ? (N + 63) / 64 : (N + 127) / 128);
+    if (grid.y > 65535) return TS_BAD_SHAPE;
+#define MOE_LDS(WM, WN, GLU, TO) \
+    moe_gemm_lds_kernel<WM, WN, GLU, TO><<<grid, WM * WN * TS_WAVE, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w, sorted, \
+                                                                                  tiles, src_div, N, K, limit, slope, shift)
+    if (glu && out_dtype == 1) MOE_LDS(4, 1, true, bf16_t);
+    else if (!glu && out_dtype == 0) MOE_LDS(2, 2, false, float);
+    else if (!glu && out_dtype == 1) MOE_LDS(2, 2, false, bf16_t);
+    else return TS_BAD_DTYPE;
+#undef MOE_LDS
+    return ts_check_launch();
+  }
   if (mfma) {
     // (a wave takes 32 columns of all the tile's rows; with the gate, 32 gate and 32 up columns)
     dim3 grid(max_tiles, (N + 127) / 128);

@@ -25,10 +25,12 @@ conv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restr
                    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots,
                    const int32_t* __restrict__ slots, int nh, int nkv, int hd, int vd_size, int taps, float temp_coef,
                    int temp_every, int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh,
-                   int64_t vd) {
+                   int64_t vd, int num_tokens, int with_values) {
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
-  const int t = blockIdx.x;
-  const int heads = nh + 2 * nkv;
+  const int heads = nh + (with_values ? 2 : 1) * nkv;       // (without: the values go through `conv_values_kernel`)
+  const int64_t item = (int64_t)blockIdx.x * SC_WAVES + wave;  // a wave per (token, head)
+  if (item >= (int64_t)num_tokens * heads) return;
+  const int t = (int)(item / heads), h = (int)(item - (int64_t)t * heads);
   const int channels = (nh + nkv) * hd + nkv * vd_size;
   const int pos = positions[t];
   const int seq = seq_of_token[t];
@@ -40,9 +42,9 @@ conv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restr
   const int page = stores ? slot / page_size : 0, off = stores ? slot - page * page_size : 0;
   float temp = 1.0f;
   if (temp_coef != 0.f) temp = 1.0f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.0f);
-  for (int h = wave; h < heads; h += SC_WAVES) {
+  {
     const bool is_q = h < nh, is_v = h >= nh + nkv;
-    if (!is_q && !stores) continue;
+    if (!is_q && !stores) return;
     const int size = is_v ? vd_size : hd;
     const int c0 = is_v ? (nh + nkv) * hd + (h - nh - nkv) * vd_size : h * hd;
     float y[SC_MAX_HD / TS_WAVE];
@@ -80,6 +82,54 @@ conv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restr
   }
 }
 
+// The values of SC_VTOK consecutive tokens of one key/value head, through LDS: the convolution is taken with the
+// lanes along a row's dimensions, and the rows are written with the lanes along the tokens, so that tokens in
+// consecutive slots of a page (whose values lie side by side there, pages holding values transposed) leave in
+// whole segments.
+#define SC_VTOK 32
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(SC_WAVES * TS_WAVE)
+conv_values_kernel(TO* __restrict__ v_cache, const TI* __restrict__ proj, int64_t row_stride, const float* __restrict__ conv_w,
+                   const float* __restrict__ state, const int32_t* __restrict__ seq_of_token,
+                   const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots,
+                   const int32_t* __restrict__ slots, int num_tokens, int channels, int v_first, int vd_size, int taps,
+                   int page_size, int64_t vp, int64_t vs, int64_t vh, int64_t vd) {
+  __shared__ float rows_s[SC_VTOK][SC_MAX_HD + 1];
+  __shared__ int slot_s[SC_VTOK], local_s[SC_VTOK], state_s[SC_VTOK];
+  const int t0 = blockIdx.x * SC_VTOK, g = blockIdx.y;
+  const int nt = min(SC_VTOK, num_tokens - t0);
+  if (threadIdx.x < nt) {
+    const int t = t0 + threadIdx.x, seq = seq_of_token[t];
+    slot_s[threadIdx.x] = slots[t];
+    local_s[threadIdx.x] = t - cu_seqlens[seq];
+    state_s[threadIdx.x] = state_slots[seq];
+  }
+  __syncthreads();
+  const int c0 = v_first + g * vd_size;
+  for (int i = threadIdx.x; i < nt * vd_size; i += SC_WAVES * TS_WAVE) {
+    const int tl = i / vd_size, d = i - tl * vd_size;
+    const int c = c0 + d, t = t0 + tl, local = local_s[tl];
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;
+      float u;
+      if (back <= local) u = Num<TI>::ld(proj + (int64_t)(t - back) * row_stride + c);
+      else u = state[((int64_t)state_s[tl] * (taps - 1) + (taps - 1 - (back - local))) * channels + c];
+      acc = fmaf(conv_w[(int64_t)c * taps + j], u, acc);
+    }
+    rows_s[tl][d] = acc;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < vd_size * SC_VTOK; i += SC_WAVES * TS_WAVE) {
+    const int d = i / SC_VTOK, tl = i - d * SC_VTOK;
+    if (tl >= nt) continue;
+    const int slot = slot_s[tl];
+    if (slot < 0) continue;
+    const int page = slot / page_size, off = slot - page * page_size;
+    Num<TO>::st(v_cache + page * vp + off * vs + (int64_t)g * vh + (int64_t)d * vd, rows_s[tl][d]);
+  }
+}
+
 // A thread per (request of the step, channel): row i of the new state is the row that lies taps - 1 - i rows
 // before the end of (old state rows, the step's rows). Ascending i reads only rows not yet overwritten.
 template <typename TI>
@@ -112,14 +162,24 @@ extern "C" int ts_conv_finish(void* q_out, void* k_cache, void* v_cache, const v
       page_size <= 0 || (taps > 1 && !state) || (temp_coef != 0.f && temp_every <= 0) ||
       row_stride < (int64_t)(nh + nkv) * hd + (int64_t)nkv * vd_size)
     return TS_BAD_SHAPE;
+  // several tokens of a step: their values leave through the tile kernel (a few tokens', with their heads)
+  const int v_tiles = k_cache && nkv > 0 && num_tokens >= 256 && nkv <= 65535;
+  const int heads = nh + (v_tiles ? 1 : 2) * nkv;
+  const int64_t blocks = ((int64_t)num_tokens * heads + SC_WAVES - 1) / SC_WAVES;
+  if (blocks > 0x7fffffff) return TS_BAD_SHAPE;
+  const int channels = (nh + nkv) * hd + nkv * vd_size;
+  dim3 v_grid((num_tokens + SC_VTOK - 1) / SC_VTOK, nkv > 0 ? nkv : 1);
 #define SC_LAUNCH(TI, TO) \
-  conv_finish_kernel<TI, TO><<<num_tokens, SC_WAVES * TS_WAVE, 0, stream>>>( \
+  conv_finish_kernel<TI, TO><<<(unsigned)blocks, SC_WAVES * TS_WAVE, 0, stream>>>( \
       (TO*)q_out, (TO*)k_cache, (TO*)v_cache, (const TI*)proj, row_stride, conv_w, state, q_norm_w, k_norm_w, eps, positions, \
       seq_of_token, cu_seqlens, state_slots, slots, nh, nkv, hd, vd_size, taps, temp_coef, temp_every, page_size, kp, ks, kh, \
-      vp, vs, vh, vd)
-  if (in_dtype == 0 && out_dtype == 0) SC_LAUNCH(float, float);
-  else if (in_dtype == 0 && out_dtype == 1) SC_LAUNCH(float, bf16_t);
-  else if (in_dtype == 1 && out_dtype == 1) SC_LAUNCH(bf16_t, bf16_t);
+      vp, vs, vh, vd, num_tokens, !v_tiles); \
+  if (v_tiles) conv_values_kernel<TI, TO><<<v_grid, SC_WAVES * TS_WAVE, 0, stream>>>( \
+      (TO*)v_cache, (const TI*)proj, row_stride, conv_w, state, seq_of_token, cu_seqlens, state_slots, slots, num_tokens, \
+      channels, (nh + nkv) * hd, vd_size, taps, page_size, vp, vs, vh, vd)
+  if (in_dtype == 0 && out_dtype == 0) { SC_LAUNCH(float, float); }
+  else if (in_dtype == 0 && out_dtype == 1) { SC_LAUNCH(float, bf16_t); }
+  else if (in_dtype == 1 && out_dtype == 1) { SC_LAUNCH(bf16_t, bf16_t); }
   else return TS_BAD_DTYPE;
 #undef SC_LAUNCH
   return ts_check_launch();

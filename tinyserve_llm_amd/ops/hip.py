@@ -1964,7 +1964,8 @@ def conv_state_update(state: torch.Tensor, proj: torch.Tensor, ctx) -> None:
 # ---- a mixture of experts ----
 
 MOE_TILE_ROWS = 16        # rows of a tile of the experts' products,
-MOE_WIDE_TILE_ROWS = 64   # or, in bfloat16, where the experts have this many rows each on average
+MOE_WIDE_TILE_ROWS = 64   # or, in bfloat16, where the experts have this many rows each on average,
+MOE_LDS_TILE_ROWS = 128   # or this many (both operands then go through LDS; reductions that are multiples of 64)
 MOE_MAX_EXPERTS = 1024
 MOE_MAX_TOP = 32
 
@@ -2000,6 +2001,8 @@ def moe_tile_rows(pairs: int, experts: int, dtype: torch.dtype, k_sizes: "tuple[
     """Rows of a tile for a step of `pairs` (token, expert) pairs: the wide tile where the matrix-core kernel
     runs (bfloat16, reductions that are multiples of 32) and an expert has that many rows on average, so
     that an expert's matrix is read once per 64 rows and not once per 16."""
+    if dtype == torch.bfloat16 and all(k % 64 == 0 for k in k_sizes) and pairs >= MOE_LDS_TILE_ROWS * experts:
+        return MOE_LDS_TILE_ROWS
     wide = dtype == torch.bfloat16 and all(k % 32 == 0 for k in k_sizes) and pairs >= MOE_WIDE_TILE_ROWS * experts
     return MOE_WIDE_TILE_ROWS if wide else MOE_TILE_ROWS
 
@@ -2007,7 +2010,7 @@ def moe_tile_rows(pairs: int, experts: int, dtype: torch.dtype, k_sizes: "tuple[
 def moe_group(ids: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS) -> ExpertTiles:
     """Groups the step's pairs by expert and cuts the groups into tiles of up to `tile_rows` rows."""
     _gpu(ids)
-    _need(tile_rows in (MOE_TILE_ROWS, MOE_WIDE_TILE_ROWS), "tiles of 16 or 64 rows")
+    _need(tile_rows in (MOE_TILE_ROWS, MOE_WIDE_TILE_ROWS, MOE_LDS_TILE_ROWS), "tiles of 16, 64 or 128 rows")
     _need(ids.dtype == torch.int32 and ids.dim() == 2 and ids.is_contiguous(), "the chosen experts must be contiguous int32 [tokens, top]")
     _need(0 < experts <= MOE_MAX_EXPERTS, lambda: f"up to {MOE_MAX_EXPERTS} experts")
     P = ids.numel()
@@ -2037,6 +2040,7 @@ def moe_gemm(x: torch.Tensor, weights: torch.Tensor, grouped: ExpertTiles, out_d
     limit, slope, shift = glu if glu is not None else (0.0, 0.0, 0.0)
     _need(grouped.tile_rows == MOE_TILE_ROWS or (x.dtype == torch.bfloat16 and x.shape[1] % 32 == 0),
           "wide tiles are the matrix-core kernel's: bfloat16, a reduction that is a multiple of 32")
+    _need(grouped.tile_rows != MOE_LDS_TILE_ROWS or x.shape[1] % 64 == 0, "tiles of 128 rows: a reduction that is a multiple of 64")
     _run("moe_gemm", library().ts_moe_gemm(_ptr(out), _code(out_dtype), _ptr(x), _code(x.dtype), _ptr(weights), _ptr(grouped.sorted),
                                            _ptr(grouped.tiles), grouped.tiles.shape[0], grouped.tile_rows, grouped.top if per_token else 1, n, x.shape[1],
                                            int(glu is not None), float(limit), float(slope), float(shift), _stream()))
