@@ -150,7 +150,7 @@ def test_convolution_norms_multiplier_cache_and_state(in_dtype, dtype, shape):
     H, G, D, V, taps, (coef, every) = shape
     C = (H + G) * D + G * V
     extra = 24                                              # (columns after the channels: a gate's)
-    lengths, page = [300, 9, 21], 8                        # (one step of more than 256 tokens: its values leave in tiles)
+    lengths, page = [300, 9, 281], 8                       # (a step of two long portions: its heads take the kernel of 16-byte pieces where they can, its values leave in tiles)
     conv = (torch.randn(C, taps) * 0.4 + 1.0 / taps).to(DEV)
     qn, kn = (1 + 0.2 * torch.randn(D)).to(DEV), (1 + 0.2 * torch.randn(D)).to(DEV)
     proj = [rounded(torch.randn(n, C + extra), in_dtype) for n in lengths]
@@ -173,7 +173,7 @@ def test_convolution_norms_multiplier_cache_and_state(in_dtype, dtype, shape):
         if G:
             want_k.append(plain.unit_rms(y[:, H * D:(H + G) * D].view(n, G, D), eps) * kn.cpu().to(F64))
             want_v.append(y[:, (H + G) * D:].view(n, G, V))
-    cuts = [[1, 2, 1, 5, 2, 289], [2, 1, 1, 1, 4], [7, 1, 13]]
+    cuts = [[1, 2, 1, 5, 2, 289], [2, 1, 1, 1, 4], [7, 1, 13, 2, 1, 257]]
     cursors, got_q = [0, 0, 0], [[], [], []]
     for step in range(max(len(c) for c in cuts)):
         live = [i for i in range(3) if step < len(cuts[i])]

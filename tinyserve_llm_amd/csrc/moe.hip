@@ -199,6 +199,7 @@ extern "C" int ts_moe_group(const int32_t* ids, int32_t* sorted, int32_t* tiles,
 }
 
 #define MOE_BM 16
+#define MOE_DIES 8
 #define MOE_BN 64
 #define MOE_KC 32
 
@@ -353,6 +354,80 @@ moe_gemm_mfma_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const b
   }
 }
 
+// Tiles of 16 rows, for steps of few tokens, where the experts' matrices are streamed once and nothing else counts:
+// a workgroup takes a tile's rows by 16 columns (with GLU: 16 gate and 16 up columns), and its four waves take a
+// quarter of K each, four k-steps' loads in flight at a time, so that a step with one token still has a thousand
+// waves asking for memory. The quarters' sums meet through LDS and are added in the waves' order: a row's result
+// depends on K alone, not on the tile or the batch it lands in.
+template <bool GLU, typename TO>
+__global__ void __launch_bounds__(MOE_THREADS)
+moe_gemm_stream_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                       const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles, int src_div, int N, int K,
+                       float limit, float slope, float shift) {
+  constexpr int SETS = GLU ? 2 : 1;
+  constexpr int WAVES = MOE_THREADS / TS_WAVE, DEPTH = 4;
+  __shared__ moe_f32x4 part_s[WAVES - 1][SETS][TS_WAVE];
+  const int tile = blockIdx.x;
+  const int rows = tiles[3 * tile + 2];
+  if (rows == 0) return;
+  const int e = tiles[3 * tile], first = tiles[3 * tile + 1];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TS_WAVE), lane = threadIdx.x & (TS_WAVE - 1);
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.y * 16;
+  const int64_t expert_rows = GLU ? 2 * (int64_t)N : N;
+  const bf16_t* we = w + (int64_t)e * expert_rows * K;
+  const int pair = sorted[first + min(r, rows - 1)];
+  const int col = min(n0 + r, N - 1);
+  const int steps = K / 32, s0 = wave * steps / WAVES, s1 = (wave + 1) * steps / WAVES;
+  const bf16_t* xp = x + (int64_t)(pair / src_div) * K + 8 * g;
+  const bf16_t* wp[SETS];
+  wp[0] = we + (int64_t)col * K + 8 * g;
+  if constexpr (GLU) wp[1] = we + (int64_t)(N + col) * K + 8 * g;
+  moe_f32x4 acc[SETS];
+#pragma unroll
+  for (int s = 0; s < SETS; ++s) acc[s] = (moe_f32x4){0.f, 0.f, 0.f, 0.f};
+  int s = s0;
+  for (; s + DEPTH <= s1; s += DEPTH) {
+    moe_u32x4 fx[DEPTH], fw[SETS][DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      fx[d] = *(const moe_u32x4*)(xp + 32 * (s + d));
+#pragma unroll
+      for (int t = 0; t < SETS; ++t) fw[t][d] = *(const moe_u32x4*)(wp[t] + 32 * (s + d));
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+      for (int t = 0; t < SETS; ++t) acc[t] = moe_mfma(fw[t][d], fx[d], acc[t]);
+  }
+  for (; s < s1; ++s) {
+    const moe_u32x4 fx = *(const moe_u32x4*)(xp + 32 * s);
+#pragma unroll
+    for (int t = 0; t < SETS; ++t) acc[t] = moe_mfma(*(const moe_u32x4*)(wp[t] + 32 * s), fx, acc[t]);
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < SETS; ++t) part_s[wave - 1][t][lane] = acc[t];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int v = 0; v < WAVES - 1; ++v)
+#pragma unroll
+    for (int t = 0; t < SETS; ++t) acc[t] += part_s[v][t][lane];
+  // lane (r, g): row r of the tile, columns n0 + 4 g .. + 3
+  if (r >= rows) return;
+  TO* orow = out + (int64_t)pair * N;
+  const int c0 = n0 + 4 * g;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    float y;
+    if constexpr (GLU) y = moe_unit(acc[0][c], acc[1][c], limit, slope, shift);
+    else y = acc[0][c];
+    if (c0 + c < N) Num<TO>::st(orow + c0 + c, y);
+  }
+}
+
 // Tiles of 128 rows, for steps that give an expert hundreds of rows: both operands go through LDS in the order the
 // matrix instruction wants them (lane (r, g) of fragment f: row 16 (f / 2) + r, elements 32 (f % 2) + 8 g .. + 7),
 // 64 of K at a time, two k-steps in flight (one in an LDS buffer being multiplied, the next in registers on its way
@@ -363,8 +438,8 @@ moe_gemm_mfma_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const b
 template <int WM, int WN, bool GLU, typename TO>
 __global__ void __launch_bounds__(WM * WN * TS_WAVE)
 moe_gemm_lds_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                    const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles, int src_div, int N, int K,
-                    float limit, float slope, float shift) {
+                    const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles, int num_tiles, int col_blocks,
+                    int src_div, int N, int K, float limit, float slope, float shift) {
   constexpr int BM = 128, BN = 128;
   constexpr int THREADS = WM * WN * TS_WAVE;
   constexpr int FX = BM / 16 * 2, FW = BN / 16 * 2;       // fragments (a kilobyte each) of a k-step of 64
@@ -372,12 +447,18 @@ moe_gemm_lds_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf
   constexpr int LX = FX * 64 / THREADS, LW = FW * 64 / THREADS;
   static_assert(!GLU || WN == 1, "a gate sum and its up sum must meet in one wave");
   __shared__ moe_u32x4 lds[2][(FX + FW) * 64];
-  const int tile = blockIdx.x;
+  // Workgroups go to the chip's eight dies in turn, each die with a cache of its own: die d takes the d-th eighth
+  // of the (tile, column block) list, column blocks innermost and tiles in the experts' order, so that the
+  // workgroups a die runs at one time share a few tiles' rows and one expert's columns in its cache.
+  const int per_die = gridDim.x / MOE_DIES;
+  const int item = (blockIdx.x % MOE_DIES) * per_die + blockIdx.x / MOE_DIES;
+  if (item >= num_tiles * col_blocks) return;
+  const int tile = item / col_blocks;
   const int rows = tiles[3 * tile + 2];
   if (rows == 0) return;
   const int e = tiles[3 * tile], first = tiles[3 * tile + 1];
   // (with GLU a workgroup's 128 columns of the product are 64 columns of y)
-  const int n0 = blockIdx.y * (GLU ? BN / 2 : BN);
+  const int n0 = (item - tile * col_blocks) * (GLU ? BN / 2 : BN);
   const int t = threadIdx.x, lane = t % TS_WAVE, r = lane % 16, g = lane / 16;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TS_WAVE), wm = wave % WM, wn = wave / WM;
   const bf16_t* we = w + (int64_t)e * (GLU ? 2 : 1) * N * K;
@@ -496,11 +577,13 @@ extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype,
   const bool mfma = x_dtype == 1 && K % 32 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0;
   if (tile_rows == 128) {
     if (!mfma || K % 64) return TS_BAD_SHAPE;
-    dim3 grid(max_tiles, glu ? (N + 63) / 64 : (N + 127) / 128);
-    if (grid.y > 65535) return TS_BAD_SHAPE;
+    const int col_blocks = glu ? (N + 63) / 64 : (N + 127) / 128;
+    const int64_t items = (int64_t)max_tiles * col_blocks;
+    if (items > 0x3fffffff) return TS_BAD_SHAPE;
+    const unsigned grid = (unsigned)((items + MOE_DIES - 1) / MOE_DIES * MOE_DIES);
 #define MOE_LDS(WM, WN, GLU, TO) \
     moe_gemm_lds_kernel<WM, WN, GLU, TO><<<grid, WM * WN * TS_WAVE, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w, sorted, \
-                                                                                  tiles, src_div, N, K, limit, slope, shift)
+                                                                                  tiles, max_tiles, col_blocks, src_div, N, K, limit, slope, shift)
     if (glu && out_dtype == 1) MOE_LDS(4, 1, true, bf16_t);
     else if (!glu && out_dtype == 0) MOE_LDS(2, 2, false, float);
     else if (!glu && out_dtype == 1) MOE_LDS(2, 2, false, bf16_t);
@@ -509,15 +592,28 @@ extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype,
     return ts_check_launch();
   }
   if (mfma) {
+    if (tile_rows == 16) {
+      dim3 grid(max_tiles, (N + 15) / 16);
+      if (grid.y > 65535) return TS_BAD_SHAPE;
+#define MOE_STREAM(GLU, TO) \
+      moe_gemm_stream_kernel<GLU, TO><<<grid, MOE_THREADS, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w, sorted, tiles, \
+                                                                        src_div, N, K, limit, slope, shift)
+      if (glu && out_dtype == 1) MOE_STREAM(true, bf16_t);
+      else if (!glu && out_dtype == 0) MOE_STREAM(false, float);
+      else if (!glu && out_dtype == 1) MOE_STREAM(false, bf16_t);
+      else return TS_BAD_DTYPE;
+#undef MOE_STREAM
+      return ts_check_launch();
+    }
     // (a wave takes 32 columns of all the tile's rows; with the gate, 32 gate and 32 up columns)
     dim3 grid(max_tiles, (N + 127) / 128);
     if (grid.y > 65535) return TS_BAD_SHAPE;
 #define MOE_MFMA(TM, GLU, TO) \
     moe_gemm_mfma_kernel<TM, 2, GLU, TO><<<grid, MOE_THREADS, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w, sorted, \
                                                                            tiles, src_div, N, K, limit, slope, shift)
-    if (glu && out_dtype == 1) { if (tile_rows == 16) MOE_MFMA(1, true, bf16_t); else MOE_MFMA(4, true, bf16_t); }
-    else if (!glu && out_dtype == 0) { if (tile_rows == 16) MOE_MFMA(1, false, float); else MOE_MFMA(4, false, float); }
-    else if (!glu && out_dtype == 1) { if (tile_rows == 16) MOE_MFMA(1, false, bf16_t); else MOE_MFMA(4, false, bf16_t); }
+    if (glu && out_dtype == 1) MOE_MFMA(4, true, bf16_t);
+    else if (!glu && out_dtype == 0) MOE_MFMA(4, false, float);
+    else if (!glu && out_dtype == 1) MOE_MFMA(4, false, bf16_t);
     else return TS_BAD_DTYPE;
 #undef MOE_MFMA
     return ts_check_launch();

@@ -82,6 +82,123 @@ conv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restr
   }
 }
 
+// The same for the q and k heads of steps of many tokens, where head sizes are multiples of eight: a thread takes
+// eight consecutive channels of a head (32 or 16 bytes a load, 16 a store), the threads of a head sit side by side
+// in a wave (a power of two of them, the last ones idle where the head's eighths are no power of two) and add
+// their squares by exchanging registers. TAPS > 0: the taps are known when the kernel is compiled.
+#define SC_PIECE 8
+#define SC_VEC_THREADS 256
+
+template <typename T> struct ScRow;
+template <> struct ScRow<float> {
+  static __device__ __forceinline__ void ld(const float* p, float (&u)[SC_PIECE]) {
+    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    u[0] = a.x; u[1] = a.y; u[2] = a.z; u[3] = a.w; u[4] = b.x; u[5] = b.y; u[6] = b.z; u[7] = b.w;
+  }
+  static __device__ __forceinline__ void st(float* p, const float (&y)[SC_PIECE]) {
+    *(float4*)p = make_float4(y[0], y[1], y[2], y[3]);
+    *(float4*)(p + 4) = make_float4(y[4], y[5], y[6], y[7]);
+  }
+};
+template <> struct ScRow<bf16_t> {
+  static __device__ __forceinline__ void ld(const bf16_t* p, float (&u)[SC_PIECE]) {
+    const uint4 a = *(const uint4*)p;
+    const uint32_t v[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      u[2 * i] = __uint_as_float(v[i] << 16);
+      u[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void st(bf16_t* p, const float (&y)[SC_PIECE]) {
+    uint4 a;
+    a.x = (uint32_t)f2bf(y[0]) | ((uint32_t)f2bf(y[1]) << 16);
+    a.y = (uint32_t)f2bf(y[2]) | ((uint32_t)f2bf(y[3]) << 16);
+    a.z = (uint32_t)f2bf(y[4]) | ((uint32_t)f2bf(y[5]) << 16);
+    a.w = (uint32_t)f2bf(y[6]) | ((uint32_t)f2bf(y[7]) << 16);
+    *(uint4*)p = a;
+  }
+};
+
+template <typename TI, typename TO, int TAPS>
+__global__ void __launch_bounds__(SC_VEC_THREADS)
+conv_finish_vec_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, const TI* __restrict__ proj, int64_t row_stride,
+                       const float* __restrict__ conv_w, const float* __restrict__ state, const float* __restrict__ q_norm_w,
+                       const float* __restrict__ k_norm_w, float eps, const int32_t* __restrict__ positions,
+                       const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ cu_seqlens,
+                       const int32_t* __restrict__ state_slots, const int32_t* __restrict__ slots, int nh, int nkv, int hd,
+                       int channels, int taps_arg, float temp_coef, int temp_every, int page_size, int64_t kp, int64_t ks,
+                       int64_t kh, int num_tokens, int group, int group_shift) {
+  const int taps = TAPS > 0 ? TAPS : taps_arg;
+  const int heads = nh + (k_cache ? nkv : 0);
+  const int64_t gid = (int64_t)blockIdx.x * SC_VEC_THREADS + threadIdx.x;
+  const int64_t head_item = gid >> group_shift;              // (token, head): all its threads leave together
+  const int piece = (int)(gid & (group - 1));
+  if (head_item >= (int64_t)num_tokens * heads) return;
+  const int t = (int)(head_item / heads), h = (int)(head_item - (int64_t)t * heads);
+  const bool is_q = h < nh;
+  const int slot = slots ? slots[t] : -1;
+  if (!is_q && slot < 0) return;
+  const bool active = piece * SC_PIECE < hd;
+  const int seq = seq_of_token[t];
+  const int local = t - cu_seqlens[seq];
+  const int c = h * hd + (active ? piece : 0) * SC_PIECE;
+  float y[SC_PIECE];
+#pragma unroll
+  for (int i = 0; i < SC_PIECE; ++i) y[i] = 0.f;
+  if (active) {
+    const float* st = taps > 1 ? state + (int64_t)state_slots[seq] * (taps - 1) * channels : nullptr;
+    if constexpr (TAPS > 0) {
+      // every row and every weight asked for before the first is used
+      float u[TAPS][SC_PIECE], wv[SC_PIECE * TAPS];
+#pragma unroll
+      for (int j = 0; j < TAPS; ++j) {
+        const int back = TAPS - 1 - j;
+        if (back <= local) ScRow<TI>::ld(proj + (int64_t)(t - back) * row_stride + c, u[j]);
+        else ScRow<float>::ld(st + (int64_t)(TAPS - 1 - (back - local)) * channels + c, u[j]);
+      }
+#pragma unroll
+      for (int i = 0; i < SC_PIECE * TAPS / 4; ++i) {
+        const float4 a = *(const float4*)(conv_w + (int64_t)c * TAPS + 4 * i);
+        wv[4 * i] = a.x; wv[4 * i + 1] = a.y; wv[4 * i + 2] = a.z; wv[4 * i + 3] = a.w;
+      }
+#pragma unroll
+      for (int j = 0; j < TAPS; ++j)
+#pragma unroll
+        for (int i = 0; i < SC_PIECE; ++i) y[i] = fmaf(wv[i * TAPS + j], u[j][i], y[i]);
+    } else {
+      for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j;
+        float u[SC_PIECE];
+        if (back <= local) ScRow<TI>::ld(proj + (int64_t)(t - back) * row_stride + c, u);
+        else ScRow<float>::ld(st + (int64_t)(taps - 1 - (back - local)) * channels + c, u);
+#pragma unroll
+        for (int i = 0; i < SC_PIECE; ++i) y[i] = fmaf(conv_w[(int64_t)(c + i) * taps + j], u[i], y[i]);
+      }
+    }
+  }
+  const float* nw = is_q ? q_norm_w : k_norm_w;
+  float scale = 1.0f;
+  if (nw) {
+    float squares = 0.f;
+#pragma unroll
+    for (int i = 0; i < SC_PIECE; ++i) squares = fmaf(y[i], y[i], squares);
+    for (int d = group >> 1; d > 0; d >>= 1) squares += __shfl_xor(squares, d, TS_WAVE);
+    scale = 1.0f / sqrtf(squares / (float)hd + eps);
+  }
+  if (!active) return;
+  if (is_q && temp_coef != 0.f) scale *= 1.0f + temp_coef * logf((float)((positions[t] + 1) / temp_every) + 1.0f);
+#pragma unroll
+  for (int i = 0; i < SC_PIECE; ++i) y[i] = y[i] * scale * (nw ? nw[piece * SC_PIECE + i] : 1.0f);
+  TO* dst;
+  if (is_q) dst = q_out + ((int64_t)t * nh + h) * hd;
+  else {
+    const int page = slot / page_size, off = slot - page * page_size;
+    dst = k_cache + page * kp + off * ks + (int64_t)(h - nh) * kh;
+  }
+  ScRow<TO>::st(dst + piece * SC_PIECE, y);
+}
+
 // The values of SC_VTOK consecutive tokens of one key/value head, through LDS: the convolution is taken with the
 // lanes along a row's dimensions, and the rows are written with the lanes along the tokens, so that tokens in
 // consecutive slots of a page (whose values lie side by side there, pages holding values transposed) leave in
@@ -169,6 +286,39 @@ extern "C" int ts_conv_finish(void* q_out, void* k_cache, void* v_cache, const v
   if (blocks > 0x7fffffff) return TS_BAD_SHAPE;
   const int channels = (nh + nkv) * hd + nkv * vd_size;
   dim3 v_grid((num_tokens + SC_VTOK - 1) / SC_VTOK, nkv > 0 ? nkv : 1);
+  // steps of many tokens whose rows and heads are whole 16-byte pieces: q and k through the kernel of eight
+  // channels a thread, the values through the tile kernel
+  const int in_piece = in_dtype == 0 ? 4 : 8;
+  const bool aligned = hd % SC_PIECE == 0 && row_stride % in_piece == 0 && channels % 4 == 0 && kp % 8 == 0 && ks % 8 == 0 &&
+                       kh % 8 == 0 && (((uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)proj | (uintptr_t)conv_w |
+                                        (uintptr_t)state | (uintptr_t)q_norm_w | (uintptr_t)k_norm_w) & 15) == 0;
+  if (aligned && num_tokens >= 256 && (v_tiles || nkv == 0 || !k_cache)) {
+    int group = 1, group_shift = 0;
+    while (group * SC_PIECE < hd) group *= 2, ++group_shift;
+    const int vec_heads = nh + (k_cache ? nkv : 0);
+    const int64_t vec_blocks = ((int64_t)num_tokens * vec_heads * group + SC_VEC_THREADS - 1) / SC_VEC_THREADS;
+    if (vec_blocks > 0x7fffffff) return TS_BAD_SHAPE;
+#define SC_VEC(TI, TO, TAPS) \
+    conv_finish_vec_kernel<TI, TO, TAPS><<<(unsigned)vec_blocks, SC_VEC_THREADS, 0, stream>>>( \
+        (TO*)q_out, (TO*)k_cache, (const TI*)proj, row_stride, conv_w, state, q_norm_w, k_norm_w, eps, positions, seq_of_token, \
+        cu_seqlens, state_slots, slots, nh, nkv, hd, channels, taps, temp_coef, temp_every, page_size, kp, ks, kh, num_tokens, \
+        group, group_shift)
+#define SC_VEC_TAPS(TI, TO) \
+    do { \
+      if (taps == 4) SC_VEC(TI, TO, 4); else if (taps == 3) SC_VEC(TI, TO, 3); else if (taps == 2) SC_VEC(TI, TO, 2); \
+      else SC_VEC(TI, TO, 0); \
+      if (v_tiles) conv_values_kernel<TI, TO><<<v_grid, SC_WAVES * TS_WAVE, 0, stream>>>( \
+          (TO*)v_cache, (const TI*)proj, row_stride, conv_w, state, seq_of_token, cu_seqlens, state_slots, slots, num_tokens, \
+          channels, (nh + nkv) * hd, vd_size, taps, page_size, vp, vs, vh, vd); \
+    } while (0)
+    if (in_dtype == 0 && out_dtype == 0) SC_VEC_TAPS(float, float);
+    else if (in_dtype == 0 && out_dtype == 1) SC_VEC_TAPS(float, bf16_t);
+    else if (in_dtype == 1 && out_dtype == 1) SC_VEC_TAPS(bf16_t, bf16_t);
+    else return TS_BAD_DTYPE;
+#undef SC_VEC_TAPS
+#undef SC_VEC
+    return ts_check_launch();
+  }
 #define SC_LAUNCH(TI, TO) \
   conv_finish_kernel<TI, TO><<<(unsigned)blocks, SC_WAVES * TS_WAVE, 0, stream>>>( \
       (TO*)q_out, (TO*)k_cache, (TO*)v_cache, (const TI*)proj, row_stride, conv_w, state, q_norm_w, k_norm_w, eps, positions, \
