@@ -173,7 +173,7 @@ def test_convolution_norms_multiplier_cache_and_state(in_dtype, dtype, shape):
         if G:
             want_k.append(plain.unit_rms(y[:, H * D:(H + G) * D].view(n, G, D), eps) * kn.cpu().to(F64))
             want_v.append(y[:, (H + G) * D:].view(n, G, V))
-    cuts = [[1, 2, 1, 5, 2, 289], [2, 1, 1, 1, 4], [7, 1, 13, 2, 1, 257]]
+    cuts = [[1, 2, 1, 2, 2, 292], [2, 1, 1, 1, 4], [7, 1, 13, 2, 1, 257]]      # (the first long portion starts at a page's first slot, the second does not)
     cursors, got_q = [0, 0, 0], [[], [], []]
     for step in range(max(len(c) for c in cuts)):
         live = [i for i in range(3) if step < len(cuts[i])]

@@ -120,6 +120,42 @@ template <> struct ScRow<bf16_t> {
   }
 };
 
+// Eight consecutive channels from c of token t's convolution; `local`: tokens of the step before it, `st`: its
+// request's state rows.
+template <typename TI, int TAPS>
+__device__ __forceinline__ void sc_conv_piece(float (&y)[SC_PIECE], const TI* __restrict__ proj, int64_t row_stride,
+                                              const float* __restrict__ conv_w, const float* __restrict__ st, int channels,
+                                              int taps, int t, int local, int c) {
+  if constexpr (TAPS > 0) {
+    // every row and every weight asked for before the first is used
+    float u[TAPS][SC_PIECE], wv[SC_PIECE * TAPS];
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) {
+      const int back = TAPS - 1 - j;
+      if (back <= local) ScRow<TI>::ld(proj + (int64_t)(t - back) * row_stride + c, u[j]);
+      else ScRow<float>::ld(st + (int64_t)(TAPS - 1 - (back - local)) * channels + c, u[j]);
+    }
+#pragma unroll
+    for (int i = 0; i < SC_PIECE * TAPS / 4; ++i) {
+      const float4 a = *(const float4*)(conv_w + (int64_t)c * TAPS + 4 * i);
+      wv[4 * i] = a.x; wv[4 * i + 1] = a.y; wv[4 * i + 2] = a.z; wv[4 * i + 3] = a.w;
+    }
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j)
+#pragma unroll
+      for (int i = 0; i < SC_PIECE; ++i) y[i] = fmaf(wv[i * TAPS + j], u[j][i], y[i]);
+  } else {
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;
+      float u[SC_PIECE];
+      if (back <= local) ScRow<TI>::ld(proj + (int64_t)(t - back) * row_stride + c, u);
+      else ScRow<float>::ld(st + (int64_t)(taps - 1 - (back - local)) * channels + c, u);
+#pragma unroll
+      for (int i = 0; i < SC_PIECE; ++i) y[i] = fmaf(conv_w[(int64_t)(c + i) * taps + j], u[i], y[i]);
+    }
+  }
+}
+
 template <typename TI, typename TO, int TAPS>
 __global__ void __launch_bounds__(SC_VEC_THREADS)
 conv_finish_vec_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, const TI* __restrict__ proj, int64_t row_stride,
@@ -146,37 +182,9 @@ conv_finish_vec_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, const T
   float y[SC_PIECE];
 #pragma unroll
   for (int i = 0; i < SC_PIECE; ++i) y[i] = 0.f;
-  if (active) {
-    const float* st = taps > 1 ? state + (int64_t)state_slots[seq] * (taps - 1) * channels : nullptr;
-    if constexpr (TAPS > 0) {
-      // every row and every weight asked for before the first is used
-      float u[TAPS][SC_PIECE], wv[SC_PIECE * TAPS];
-#pragma unroll
-      for (int j = 0; j < TAPS; ++j) {
-        const int back = TAPS - 1 - j;
-        if (back <= local) ScRow<TI>::ld(proj + (int64_t)(t - back) * row_stride + c, u[j]);
-        else ScRow<float>::ld(st + (int64_t)(TAPS - 1 - (back - local)) * channels + c, u[j]);
-      }
-#pragma unroll
-      for (int i = 0; i < SC_PIECE * TAPS / 4; ++i) {
-        const float4 a = *(const float4*)(conv_w + (int64_t)c * TAPS + 4 * i);
-        wv[4 * i] = a.x; wv[4 * i + 1] = a.y; wv[4 * i + 2] = a.z; wv[4 * i + 3] = a.w;
-      }
-#pragma unroll
-      for (int j = 0; j < TAPS; ++j)
-#pragma unroll
-        for (int i = 0; i < SC_PIECE; ++i) y[i] = fmaf(wv[i * TAPS + j], u[j][i], y[i]);
-    } else {
-      for (int j = 0; j < taps; ++j) {
-        const int back = taps - 1 - j;
-        float u[SC_PIECE];
-        if (back <= local) ScRow<TI>::ld(proj + (int64_t)(t - back) * row_stride + c, u);
-        else ScRow<float>::ld(st + (int64_t)(taps - 1 - (back - local)) * channels + c, u);
-#pragma unroll
-        for (int i = 0; i < SC_PIECE; ++i) y[i] = fmaf(conv_w[(int64_t)(c + i) * taps + j], u[i], y[i]);
-      }
-    }
-  }
+  if (active)
+    sc_conv_piece<TI, TAPS>(y, proj, row_stride, conv_w, taps > 1 ? state + (int64_t)state_slots[seq] * (taps - 1) * channels : nullptr,
+                            channels, taps, t, local, c);
   const float* nw = is_q ? q_norm_w : k_norm_w;
   float scale = 1.0f;
   if (nw) {
@@ -247,6 +255,66 @@ conv_values_kernel(TO* __restrict__ v_cache, const TI* __restrict__ proj, int64_
   }
 }
 
+// The same in 16-byte pieces, where a value head is whole eighths and the cache keeps a page's slots side by side:
+// a thread convolves eight channels of a token, and writes eight tokens of a channel, in one store where their
+// slots are eight in a row from a multiple of eight.
+template <typename TI, typename TO, int TAPS>
+__global__ void __launch_bounds__(SC_VEC_THREADS)
+conv_values_vec_kernel(TO* __restrict__ v_cache, const TI* __restrict__ proj, int64_t row_stride, const float* __restrict__ conv_w,
+                       const float* __restrict__ state, const int32_t* __restrict__ seq_of_token,
+                       const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots,
+                       const int32_t* __restrict__ slots, int num_tokens, int channels, int v_first, int vd_size, int taps_arg,
+                       int page_size, int64_t vp, int64_t vh, int64_t vd) {
+  __shared__ float rows_s[SC_VTOK][SC_MAX_HD + 1];
+  __shared__ int slot_s[SC_VTOK], local_s[SC_VTOK], state_s[SC_VTOK];
+  const int taps = TAPS > 0 ? TAPS : taps_arg;
+  const int t0 = blockIdx.x * SC_VTOK, g = blockIdx.y;
+  const int nt = min(SC_VTOK, num_tokens - t0);
+  if (threadIdx.x < SC_VTOK) {
+    const int t = t0 + threadIdx.x;
+    const int seq = threadIdx.x < nt ? seq_of_token[t] : 0;
+    slot_s[threadIdx.x] = threadIdx.x < nt ? slots[t] : -1;
+    local_s[threadIdx.x] = threadIdx.x < nt ? t - cu_seqlens[seq] : 0;
+    state_s[threadIdx.x] = threadIdx.x < nt ? state_slots[seq] : 0;
+  }
+  __syncthreads();
+  const int c0 = v_first + g * vd_size, pieces = vd_size / SC_PIECE;
+  for (int i = threadIdx.x; i < nt * pieces; i += SC_VEC_THREADS) {
+    const int tl = i / pieces, piece = i - tl * pieces;
+    float y[SC_PIECE];
+#pragma unroll
+    for (int k = 0; k < SC_PIECE; ++k) y[k] = 0.f;
+    sc_conv_piece<TI, TAPS>(y, proj, row_stride, conv_w, taps > 1 ? state + (int64_t)state_s[tl] * (taps - 1) * channels : nullptr,
+                            channels, taps, t0 + tl, local_s[tl], c0 + piece * SC_PIECE);
+#pragma unroll
+    for (int k = 0; k < SC_PIECE; ++k) rows_s[tl][piece * SC_PIECE + k] = y[k];
+  }
+  __syncthreads();
+  constexpr int RUNS = SC_VTOK / SC_PIECE;                 // runs of eight tokens
+  for (int i = threadIdx.x; i < vd_size * RUNS; i += SC_VEC_THREADS) {
+    const int d = i / RUNS, run = i - d * RUNS, tl0 = run * SC_PIECE;
+    if (tl0 >= nt) continue;
+    const int first = slot_s[tl0];
+    bool row = first >= 0 && first % SC_PIECE == 0 && first % page_size + SC_PIECE <= page_size && tl0 + SC_PIECE <= nt;
+#pragma unroll
+    for (int k = 1; k < SC_PIECE; ++k) row = row && slot_s[min(tl0 + k, SC_VTOK - 1)] == first + k;
+    if (row) {
+      float y[SC_PIECE];
+#pragma unroll
+      for (int k = 0; k < SC_PIECE; ++k) y[k] = rows_s[tl0 + k][d];
+      const int page = first / page_size, off = first - page * page_size;
+      ScRow<TO>::st(v_cache + page * vp + off + (int64_t)g * vh + (int64_t)d * vd, y);
+    } else {
+      for (int k = 0; k < SC_PIECE && tl0 + k < nt; ++k) {
+        const int slot = slot_s[tl0 + k];
+        if (slot < 0) continue;
+        const int page = slot / page_size, off = slot - page * page_size;
+        Num<TO>::st(v_cache + page * vp + off + (int64_t)g * vh + (int64_t)d * vd, rows_s[tl0 + k][d]);
+      }
+    }
+  }
+}
+
 // A thread per (request of the step, channel): row i of the new state is the row that lies taps - 1 - i rows
 // before the end of (old state rows, the step's rows). Ascending i reads only rows not yet overwritten.
 template <typename TI>
@@ -303,11 +371,21 @@ extern "C" int ts_conv_finish(void* q_out, void* k_cache, void* v_cache, const v
         (TO*)q_out, (TO*)k_cache, (const TI*)proj, row_stride, conv_w, state, q_norm_w, k_norm_w, eps, positions, seq_of_token, \
         cu_seqlens, state_slots, slots, nh, nkv, hd, channels, taps, temp_coef, temp_every, page_size, kp, ks, kh, num_tokens, \
         group, group_shift)
+#define SC_VAL(TI, TO, TAPS) \
+    conv_values_vec_kernel<TI, TO, TAPS><<<v_grid, SC_VEC_THREADS, 0, stream>>>( \
+        (TO*)v_cache, (const TI*)proj, row_stride, conv_w, state, seq_of_token, cu_seqlens, state_slots, slots, num_tokens, \
+        channels, (nh + nkv) * hd, vd_size, taps, page_size, vp, vh, vd)
+    // (values whose heads are whole eighths, in a cache whose pages keep their slots side by side)
+    const bool v_pieces = vd_size % SC_PIECE == 0 && vs == 1 && page_size % SC_PIECE == 0 && vp % 8 == 0 && vh % 8 == 0 &&
+                          vd % 8 == 0 && ((uintptr_t)v_cache & 15) == 0;
 #define SC_VEC_TAPS(TI, TO) \
     do { \
       if (taps == 4) SC_VEC(TI, TO, 4); else if (taps == 3) SC_VEC(TI, TO, 3); else if (taps == 2) SC_VEC(TI, TO, 2); \
       else SC_VEC(TI, TO, 0); \
-      if (v_tiles) conv_values_kernel<TI, TO><<<v_grid, SC_WAVES * TS_WAVE, 0, stream>>>( \
+      if (v_tiles && v_pieces) { \
+        if (taps == 4) SC_VAL(TI, TO, 4); else if (taps == 3) SC_VAL(TI, TO, 3); else if (taps == 2) SC_VAL(TI, TO, 2); \
+        else SC_VAL(TI, TO, 0); \
+      } else if (v_tiles) conv_values_kernel<TI, TO><<<v_grid, SC_WAVES * TS_WAVE, 0, stream>>>( \
           (TO*)v_cache, (const TI*)proj, row_stride, conv_w, state, seq_of_token, cu_seqlens, state_slots, slots, num_tokens, \
           channels, (nh + nkv) * hd, vd_size, taps, page_size, vp, vs, vh, vd); \
     } while (0)
@@ -316,6 +394,7 @@ extern "C" int ts_conv_finish(void* q_out, void* k_cache, void* v_cache, const v
     else if (in_dtype == 1 && out_dtype == 1) SC_VEC_TAPS(bf16_t, bf16_t);
     else return TS_BAD_DTYPE;
 #undef SC_VEC_TAPS
+#undef SC_VAL
 #undef SC_VEC
     return ts_check_launch();
   }
