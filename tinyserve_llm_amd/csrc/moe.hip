@@ -632,15 +632,37 @@ extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype,
   return ts_check_launch();
 }
 
+// A thread per four columns of a token (or per column, where rows are no whole 16-byte pieces): a step of one token
+// spreads over the row's width and waits for memory once.
+template <int VEC>
 __global__ void __launch_bounds__(MOE_THREADS)
 moe_combine_kernel(float* __restrict__ out, const float* __restrict__ rows, const float* __restrict__ weights,
                    const float* __restrict__ shared, int width, int top) {
   const int64_t t = blockIdx.x;
-  for (int i = threadIdx.x; i < width; i += MOE_THREADS) {
-    float acc = 0.f;
-    for (int j = 0; j < top; ++j) acc = fmaf(weights[t * top + j], rows[(t * top + j) * width + i], acc);
-    if (shared) acc += shared[t * width + i];
-    out[t * width + i] = acc;
+  const int i = (blockIdx.y * MOE_THREADS + threadIdx.x) * VEC;
+  if (i >= width) return;
+  float acc[VEC];
+#pragma unroll
+  for (int c = 0; c < VEC; ++c) acc[c] = 0.f;
+  for (int j = 0; j < top; ++j) {
+    const float w = weights[t * top + j];
+    const float* row = rows + (t * top + j) * width + i;
+    if constexpr (VEC == 4) {
+      const float4 v = *(const float4*)row;
+      acc[0] = fmaf(w, v.x, acc[0]); acc[1] = fmaf(w, v.y, acc[1]); acc[2] = fmaf(w, v.z, acc[2]); acc[3] = fmaf(w, v.w, acc[3]);
+    } else {
+      acc[0] = fmaf(w, row[0], acc[0]);
+    }
+  }
+  if constexpr (VEC == 4) {
+    if (shared) {
+      const float4 v = *(const float4*)(shared + t * width + i);
+      acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+    }
+    *(float4*)(out + t * width + i) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+  } else {
+    if (shared) acc[0] += shared[t * width + i];
+    out[t * width + i] = acc[0];
   }
 }
 
@@ -648,6 +670,11 @@ extern "C" int ts_moe_combine(float* out, const float* rows, const float* weight
                               int width, int top, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (width <= 0 || top <= 0) return TS_BAD_SHAPE;
-  moe_combine_kernel<<<num_tokens, MOE_THREADS, 0, stream>>>(out, rows, weights, shared, width, top);
+  const bool by4 = width % 4 == 0 && (((uintptr_t)out | (uintptr_t)rows | (uintptr_t)shared) & 15) == 0;
+  const int per_block = MOE_THREADS * (by4 ? 4 : 1);
+  dim3 grid(num_tokens, (width + per_block - 1) / per_block);
+  if (grid.y > 65535) return TS_BAD_SHAPE;
+  if (by4) moe_combine_kernel<4><<<grid, MOE_THREADS, 0, stream>>>(out, rows, weights, shared, width, top);
+  else moe_combine_kernel<1><<<grid, MOE_THREADS, 0, stream>>>(out, rows, weights, shared, width, top);
   return ts_check_launch();
 }
