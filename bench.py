@@ -521,9 +521,11 @@ def fanotar(args) -> int:
             us_r = timed(lambda: hip.qkv_finish(plain32, freqs, ctx.positions, slots, k, v, nh, nkv, hd, hd, bf, qk_norm_eps=1e-5, v_norm_eps=1e-5))
 
             def finish():
+                fused = hip.conv_moves_state(ctx)              # (steps of single tokens: the state moves on in the same launch)
                 out = hip.conv_finish(qkv32, conv, state, ctx, slots, k, v, nh, nkv, hd, hd, bf, q_norm=nw, k_norm=nw, eps=1e-5,
-                                      temp_coef=0.1, temp_every=1024)
-                hip.conv_state_update(state, qkv32, ctx)
+                                      temp_coef=0.1, temp_every=1024, moves_state=fused)
+                if not fused:
+                    hip.conv_state_update(state, qkv32, ctx)
                 return out
             us_f = timed(finish)
             nbytes = T * row * (4 + 2)

@@ -173,7 +173,7 @@ def test_convolution_norms_multiplier_cache_and_state(in_dtype, dtype, shape):
         if G:
             want_k.append(plain.unit_rms(y[:, H * D:(H + G) * D].view(n, G, D), eps) * kn.cpu().to(F64))
             want_v.append(y[:, (H + G) * D:].view(n, G, V))
-    cuts = [[1, 2, 1, 2, 2, 292], [2, 1, 1, 1, 4], [7, 1, 13, 2, 1, 257]]      # (the first long portion starts at a page's first slot, the second does not)
+    cuts = [[1, 2, 1, 2, 2, 292], [2, 1, 1, 1, 4], [7, 1, 1, 12, 3, 257]]      # (the first long portion starts at a page's first slot, the second does not)
     cursors, got_q = [0, 0, 0], [[], [], []]
     for step in range(max(len(c) for c in cuts)):
         live = [i for i in range(3) if step < len(cuts[i])]
@@ -182,8 +182,10 @@ def test_convolution_norms_multiplier_cache_and_state(in_dtype, dtype, shape):
         ctx = step_context([tables[i] for i in live], page, starts, counts, [slots[i] for i in live])
         rows = torch.cat([proj[i][0][cursors[i]:cursors[i] + cuts[i][step]] for i in live])
         q = h.conv_finish(rows, conv, state, ctx, ctx.slot_mapping[0] if G else None, k if G else None, v if G else None, H, G, D, V,
-                          dtype, q_norm=qn, k_norm=kn if G else None, eps=eps, temp_coef=coef, temp_every=every)
-        if taps > 1:
+                          dtype, q_norm=qn, k_norm=kn if G else None, eps=eps, temp_coef=coef, temp_every=every,
+                          moves_state=(fused := taps > 1 and h.conv_moves_state(ctx)))
+        assert fused == (taps > 1 and set(counts) == {1})     # (the third step: a token of each request)
+        if taps > 1 and not fused:
             h.conv_state_update(state, rows, ctx)
         at = 0
         for i, n in zip(live, counts):

@@ -15,17 +15,18 @@
 #define SC_WAVES 4
 #define SC_MAX_HD 256
 #define SC_MAX_TAPS 16
+#define SC_LONG_STEP 256      // tokens from which a step's heads and values take the kernels of 16-byte pieces and tiles
 
 template <typename TI, typename TO>
 __global__ void __launch_bounds__(SC_WAVES * TS_WAVE)
 conv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restrict__ v_cache, const TI* __restrict__ proj,
-                   int64_t row_stride, const float* __restrict__ conv_w, const float* __restrict__ state,
+                   int64_t row_stride, const float* __restrict__ conv_w, float* state,
                    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
                    const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
                    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots,
                    const int32_t* __restrict__ slots, int nh, int nkv, int hd, int vd_size, int taps, float temp_coef,
                    int temp_every, int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh,
-                   int64_t vd, int num_tokens, int with_values) {
+                   int64_t vd, int num_tokens, int with_values, int moves_state) {
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
   const int heads = nh + (with_values ? 2 : 1) * nkv;       // (without: the values go through `conv_values_kernel`)
   const int64_t item = (int64_t)blockIdx.x * SC_WAVES + wave;  // a wave per (token, head)
@@ -36,7 +37,7 @@ conv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restr
   const int seq = seq_of_token[t];
   const int first = cu_seqlens[seq];                   // the step's first token of this request
   const int local = t - first;                         // tokens of the step before this one
-  const float* st = taps > 1 ? state + (int64_t)state_slots[seq] * (taps - 1) * channels : nullptr;
+  float* st = taps > 1 ? state + (int64_t)state_slots[seq] * (taps - 1) * channels : nullptr;
   const int slot = slots ? slots[t] : -1;
   const bool stores = slot >= 0 && k_cache;
   const int page = stores ? slot / page_size : 0, off = stores ? slot - page * page_size : 0;
@@ -61,6 +62,9 @@ conv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restr
           if (back <= local) u = Num<TI>::ld(proj + (int64_t)(t - back) * row_stride + c);
           else u = st[(int64_t)(taps - 1 - (back - local)) * channels + c];
           acc = fmaf(conv_w[(int64_t)c * taps + j], u, acc);
+          // a step of single tokens: this thread alone reads the channel's past rows, and moves them on by the
+          // token's own row as it goes (row j - 1 has been read when row j is written over it)
+          if (moves_state && j > 0) st[(int64_t)(j - 1) * channels + c] = u;
         }
       }
       y[i] = acc;
@@ -336,19 +340,22 @@ conv_state_update_kernel(float* __restrict__ state, const TI* __restrict__ proj,
 }
 
 extern "C" int ts_conv_finish(void* q_out, void* k_cache, void* v_cache, const void* proj, int64_t row_stride,
-                              const float* conv_w, const float* state, const float* q_norm_w, const float* k_norm_w, float eps,
+                              const float* conv_w, float* state, const float* q_norm_w, const float* k_norm_w, float eps,
                               const int32_t* positions, const int32_t* seq_of_token, const int32_t* cu_seqlens,
                               const int32_t* state_slots, const int32_t* slots, int num_tokens, int nh, int nkv, int hd,
                               int vd_size, int taps, float temp_coef, int temp_every, int page_size, int64_t kp, int64_t ks,
                               int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int in_dtype, int out_dtype,
-                              hipStream_t stream) {
+                              int moves_state, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
+  // (the state moves on inside this launch only where every request of the step feeds one token and the kernel of
+  // a wave per head takes all channels: the caller asks for it on those steps alone)
+  if (moves_state && (num_tokens >= SC_LONG_STEP || taps < 2)) return TS_BAD_SHAPE;
   if (hd <= 0 || hd > SC_MAX_HD || vd_size <= 0 || vd_size > SC_MAX_HD || nh <= 0 || nkv < 0 || taps < 1 || taps > SC_MAX_TAPS ||
       page_size <= 0 || (taps > 1 && !state) || (temp_coef != 0.f && temp_every <= 0) ||
       row_stride < (int64_t)(nh + nkv) * hd + (int64_t)nkv * vd_size)
     return TS_BAD_SHAPE;
   // several tokens of a step: their values leave through the tile kernel (a few tokens', with their heads)
-  const int v_tiles = k_cache && nkv > 0 && num_tokens >= 256 && nkv <= 65535;
+  const int v_tiles = k_cache && nkv > 0 && num_tokens >= SC_LONG_STEP && nkv <= 65535;
   const int heads = nh + (v_tiles ? 1 : 2) * nkv;
   const int64_t blocks = ((int64_t)num_tokens * heads + SC_WAVES - 1) / SC_WAVES;
   if (blocks > 0x7fffffff) return TS_BAD_SHAPE;
@@ -360,7 +367,7 @@ extern "C" int ts_conv_finish(void* q_out, void* k_cache, void* v_cache, const v
   const bool aligned = hd % SC_PIECE == 0 && row_stride % in_piece == 0 && channels % 4 == 0 && kp % 8 == 0 && ks % 8 == 0 &&
                        kh % 8 == 0 && (((uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)proj | (uintptr_t)conv_w |
                                         (uintptr_t)state | (uintptr_t)q_norm_w | (uintptr_t)k_norm_w) & 15) == 0;
-  if (aligned && num_tokens >= 256 && (v_tiles || nkv == 0 || !k_cache)) {
+  if (aligned && num_tokens >= SC_LONG_STEP && (v_tiles || nkv == 0 || !k_cache)) {
     int group = 1, group_shift = 0;
     while (group * SC_PIECE < hd) group *= 2, ++group_shift;
     const int vec_heads = nh + (k_cache ? nkv : 0);
@@ -402,7 +409,7 @@ extern "C" int ts_conv_finish(void* q_out, void* k_cache, void* v_cache, const v
   conv_finish_kernel<TI, TO><<<(unsigned)blocks, SC_WAVES * TS_WAVE, 0, stream>>>( \
       (TO*)q_out, (TO*)k_cache, (TO*)v_cache, (const TI*)proj, row_stride, conv_w, state, q_norm_w, k_norm_w, eps, positions, \
       seq_of_token, cu_seqlens, state_slots, slots, nh, nkv, hd, vd_size, taps, temp_coef, temp_every, page_size, kp, ks, kh, \
-      vp, vs, vh, vd, num_tokens, !v_tiles); \
+      vp, vs, vh, vd, num_tokens, !v_tiles, moves_state); \
   if (v_tiles) conv_values_kernel<TI, TO><<<v_grid, SC_WAVES * TS_WAVE, 0, stream>>>( \
       (TO*)v_cache, (const TI*)proj, row_stride, conv_w, state, seq_of_token, cu_seqlens, state_slots, slots, num_tokens, \
       channels, (nh + nkv) * hd, vd_size, taps, page_size, vp, vs, vh, vd)

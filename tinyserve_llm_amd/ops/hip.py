@@ -92,7 +92,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_embedding_dyt_stream": [p, p, i, p, f, p, p, p, i, i, p],
         "ts_capped_glu": [p, i, p, i, i64, i, i, f, f, f, p],
         "ts_conv_finish": [p, p, p, p, i64, p, p, p, p, f, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i64, i64, i64, i64, i64,
-                           i64, i64, i, i, p],
+                           i64, i64, i, i, i, p],
         "ts_conv_state_update": [p, p, i64, p, p, i, i, i, i, p],
         "ts_moe_route": [p, p, p, i, p, p, i, i, i, i, f, i, p],
         "ts_moe_group": [p, p, p, i, i, i, i, p],
@@ -1903,14 +1903,15 @@ CONV_MAX_TAPS = 16
 def conv_finish(proj: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor | None, ctx, slots: torch.Tensor | None,
                 k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, num_heads: int, num_kv_heads: int, head_dim: int,
                 value_dim: int, out_dtype: torch.dtype, *, q_norm: torch.Tensor | None = None, k_norm: torch.Tensor | None = None,
-                eps: float = 0.0, temp_coef: float = 0.0, temp_every: int = 1) -> torch.Tensor:
+                eps: float = 0.0, temp_coef: float = 0.0, temp_every: int = 1, moves_state: bool = False) -> torch.Tensor:
     """From projected rows (float32 or `out_dtype`, [tokens, >= channels], the channels q | k | v leading each
     row; `num_kv_heads` 0: q only) to q [tokens, heads, head_dim] and the cache slots of k and v: every channel
     first passes the causal convolution y_t = sum_j conv_w[c, j] u_(t - taps + 1 + j) over its request's rows,
     those before the step taken from `state` ([slots, taps - 1, channels] float32, oldest first); then q and k
     heads are divided by their root mean square and scaled by `q_norm` / `k_norm` ([head_dim] float32; None:
     not), and q is multiplied by 1 + temp_coef ln(floor((p + 1) / temp_every) + 1). The state is moved on by
-    `conv_state_update`, which the caller runs after this."""
+    `conv_state_update`, which the caller runs after this; or, with `moves_state`, by this launch itself, which
+    a step allows whose requests feed one token each (`conv_moves_state(ctx)`)."""
     _gpu(proj, conv_w, state, slots, k_cache, v_cache, q_norm, k_norm)
     T = proj.shape[0]
     channels = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
@@ -1938,13 +1939,25 @@ def conv_finish(proj: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor | 
         page_size, kst, vst = k_cache.shape[1], k_cache.stride()[:3], v_cache.stride()
     else:
         _need(num_kv_heads == 0, "key and value channels need a cache to go to")
+    _need(not moves_state or (taps > 1 and conv_moves_state(ctx)), "the state moves on with the heads only in steps of single tokens")
     q = torch.empty((T, num_heads, head_dim), dtype=out_dtype, device=proj.device)
     _run("conv_finish", library().ts_conv_finish(
         _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(proj), proj.stride(0), _ptr(conv_w), _ptr(state), _ptr(q_norm), _ptr(k_norm),
         float(eps), _ptr(ctx.positions), _ptr(ctx.seq_of_token), _ptr(ctx.cu_seqlens), _ptr(ctx.state_slots), _ptr(slots), T,
         num_heads, num_kv_heads, head_dim, value_dim, taps, float(temp_coef), int(temp_every), page_size, *kst, *vst,
-        _code(proj.dtype), _code(out_dtype), _stream()))
+        _code(proj.dtype), _code(out_dtype), int(moves_state), _stream()))
     return q
+
+
+CONV_LONG_STEP = 256     # tokens from which a step takes the kernels of 16-byte pieces and tiles
+
+
+def conv_moves_state(ctx) -> bool:
+    """Whether `conv_finish` may move the state on itself: every request of the step feeds exactly one token
+    (then one thread alone reads and writes a channel's past rows), and the step is short enough for the
+    kernel that takes all channels in one launch."""
+    return ctx.num_tokens == ctx.num_seqs and ctx.num_tokens < CONV_LONG_STEP and all(
+        b - a == 1 for a, b in zip(ctx.host_cu_seqlens, ctx.host_cu_seqlens[1:]))
 
 
 def conv_state_update(state: torch.Tensor, proj: torch.Tensor, ctx) -> None:

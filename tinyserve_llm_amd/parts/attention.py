@@ -288,8 +288,9 @@ class ConvAttention(Mixer):
         store = (ctx.slot_mapping[mem.space], mem.k_cache, mem.v_cache) if self.own_kv else (None, None, None)
         q = hip.conv_finish(proj, self.conv, mem.state, ctx, *store, self.num_heads, self.num_kv_heads if self.own_kv else 0,
                             self.head_dim, self.value_dim, x.dtype, q_norm=self.q_norm, k_norm=self.k_norm,
-                            eps=self.qk_norm_eps or 0.0, temp_coef=self.q_temp_coef, temp_every=self.q_temp_every)
-        if self.conv_taps > 1:
+                            eps=self.qk_norm_eps or 0.0, temp_coef=self.q_temp_coef, temp_every=self.q_temp_every,
+                            moves_state=(fused := self.conv_taps > 1 and hip.conv_moves_state(ctx)))
+        if self.conv_taps > 1 and not fused:
             hip.conv_state_update(mem.state, proj, ctx)
         o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window, sinks=self.sink,
                                 slopes=self.slopes, gate=proj[:, self.channels:] if self.has_gate else None)
