@@ -33,10 +33,11 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
                         const int32_t* __restrict__ positions, int nh, int G, int page_size, int page_shift, int page_run,
                         int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
                         int num_splits, int chunk, float scale2, int window, float cap_in, float cap_out, int sink,
-                        const float* __restrict__ sinks, const float* __restrict__ slopes) {
+                        const float* __restrict__ sinks, const float* __restrict__ slopes, const float* __restrict__ gate,
+                        int64_t gate_stride) {
   constexpr int NC = HD / 32;    // 32-dimension pieces of a key row (one 16-byte load per lane each)
   constexpr int NDB = HD / 16;   // 16-dimension blocks of the output
-  ts_fetch_arguments<GENERAL ? 176 : 164>();     // (nine pointers, five numbers, six strides, four more numbers and the scale; the caps and the sink)
+  ts_fetch_arguments<GENERAL ? 192 : 164>();     // (nine pointers, five numbers, six strides, four more numbers and the scale; the caps, the sink and the gate)
   extern __shared__ __align__(16) float smem[];
   const int nw = blockDim.x / TS_WAVE;
   float* wm = smem;                       // [waves][16]
@@ -129,7 +130,9 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
     }
     if (num_splits == 1) {                  // the whole context was this workgroup's: position `pos` is always visible
       if (GENERAL && sink) L += fast_exp2((sinks ? sinks[kvh * G + head] * 1.44269504088896340736f : 0.f) - M);
-      out[((int64_t)t * nh + (int64_t)kvh * G + head) * HD + d] = f2bf(acc / L);
+      float y = acc / L;
+      if (GENERAL) y *= ts_out_gate(gate, (int64_t)t * gate_stride + ((int64_t)kvh * G + head) * HD + d);
+      out[((int64_t)t * nh + (int64_t)kvh * G + head) * HD + d] = f2bf(y);
     } else {
       const int64_t row = ((int64_t)t * nh + (int64_t)kvh * G + head) * num_splits + split;
       part_o[row * HD + d] = acc;
@@ -146,7 +149,8 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
 __global__ void __launch_bounds__(TS_WAVE)
 attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                            const float* __restrict__ part_ml, const int32_t* __restrict__ positions, int nh, int hd,
-                           int num_splits, int chunk, int window, int sink, const float* __restrict__ sinks) {
+                           int num_splits, int chunk, int window, int sink, const float* __restrict__ sinks,
+                           const float* __restrict__ gate, int64_t gate_stride) {
   __shared__ float wgt[COMBINE_MAX_SPLITS];
   const int t = blockIdx.x / nh, lane = threadIdx.x;
   const int64_t th = blockIdx.x;
@@ -173,7 +177,7 @@ attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ p
     float acc = 0.f;
 #pragma unroll 4
     for (int s = 0; s <= s1 - s0; ++s) acc = fmaf(po[(int64_t)s * hd + d], wgt[s], acc);
-    out[th * hd + d] = f2bf(acc * inv);
+    out[th * hd + d] = f2bf(acc * inv * ts_out_gate(gate, (int64_t)t * gate_stride + (int64_t)(blockIdx.x % nh) * hd + d));
   }
 }
 
@@ -189,10 +193,10 @@ extern "C" int ts_attention_combine(void* out, const float* part_o, const float*
 // The combining kernel alone, for the prefill kernel's split walks (declared in attention_mfma.h).
 int ts_launch_attention_combine(void* out, const float* part_o, const float* part_ml, const int32_t* positions,
                                 int num_tokens, int nh, int hd, int num_splits, int chunk, int window,
-                                hipStream_t stream, int sink, const float* sinks) {
+                                hipStream_t stream, int sink, const float* sinks, const float* gate, int64_t gate_stride) {
   if (num_splits > COMBINE_MAX_SPLITS) return TS_BAD_SHAPE;
   attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,
-                                                                      num_splits, chunk, window, sink, sinks);
+                                                                      num_splits, chunk, window, sink, sinks, gate, gate_stride);
   return ts_check_launch();
 }
 
@@ -210,8 +214,9 @@ static int launch_decode(void* out, float* part_o, float* part_ml, const void* q
                          int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
                          int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits, int chunk,
                          int waves, float scale, int window, int page_run, int combine, bool general, float softcap, int sink,
-                         const float* sinks, const float* slopes, hipStream_t stream) {
+                         const float* sinks, const float* slopes, const float* gate, int64_t gate_stride, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
+  if (gate && (!general || !combine || gate_stride < (int64_t)nh * hd)) return TS_BAD_SHAPE;
   if (nkv <= 0 || nh % nkv || page_size <= 0 || page_size % 8 || max_blocks <= 0 || num_splits <= 0 || page_run < 0 || page_run > 16)
     return TS_BAD_SHAPE;
   if (waves < 1 || waves > DEC_WAVES_FOR(hd, chunk == 32 * waves) || chunk <= 0 || chunk % (32 * waves) || num_splits > COMBINE_MAX_SPLITS)
@@ -239,7 +244,7 @@ static int launch_decode(void* out, float* part_o, float* part_ml, const void* q
   attn_decode_mfma_kernel<HH, ON, GG><<<grid, waves * TS_WAVE, smem, stream>>>(                                 \
       (bf16_t*)out, part_o, part_ml, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,          \
       block_tables, seq_of_token, positions, nh, G, page_size, page_shift, page_run, kp, ks, kh, vp, vh, vd, max_blocks,  \
-      num_splits, chunk, scale2, window, cap_in, cap_out, sink, sinks, slopes)
+      num_splits, chunk, scale2, window, cap_in, cap_out, sink, sinks, slopes, gate, gate_stride)
 #define TS_DEC1(HH, ON) if (general) TS_DEC2(HH, ON, true); else TS_DEC2(HH, ON, false)
 #define TS_DEC(HH) if (chunk == 32 * waves) { TS_DEC1(HH, true); } else { TS_DEC1(HH, false); }
   switch (hd) {
@@ -256,7 +261,7 @@ static int launch_decode(void* out, float* part_o, float* part_ml, const void* q
   if (rc || num_splits == 1 || !combine) return rc;     // (combine 0: the caller's next kernel reads the parts itself)
   attn_decode_combine_kernel<<<num_tokens * nh, TS_WAVE, 0, stream>>>((bf16_t*)out, part_o, part_ml, positions, nh, hd,
                                                                       num_splits, chunk, window, general ? sink : 0,
-                                                                      general ? sinks : nullptr);
+                                                                      general ? sinks : nullptr, gate, gate_stride);
   return ts_check_launch();
 }
 
@@ -268,21 +273,23 @@ extern "C" int ts_paged_attention_decode(void* out, float* part_o, float* part_m
                                          int waves, float scale, int window, int page_run, int combine, hipStream_t stream) {
   return launch_decode(out, part_o, part_ml, q, k_cache, v_cache, block_tables, seq_of_token, positions, num_tokens, nh, nkv, hd,
                        page_size, kp, ks, kh, vp, vh, vd, max_blocks, num_splits, chunk, waves, scale, window, page_run, combine,
-                       false, 0.f, 0, nullptr, nullptr, stream);
+                       false, 0.f, 0, nullptr, nullptr, nullptr, 0, stream);
 }
 
 // The same with capped scores (softcap > 0: cap * tanh(score / cap)), a sink (one more in the softmax's
 // denominator; `sinks`, float [nh], if given: exp(sinks[head]) more instead), a penalty of slopes[head] (float [nh],
 // if given) per position of distance taken off every score, and weights carried in two bfloat16 terms; always combines.
+// `gate` (float [tokens, >= nh hd], rows gate_stride apart; may be null): the output leaves multiplied by sigmoid(gate).
 extern "C" int ts_paged_attention_decode_general(void* out, float* part_o, float* part_ml, const void* q, const void* k_cache,
                                                  const void* v_cache, const int32_t* block_tables,
                                                  const int32_t* seq_of_token, const int32_t* positions, int num_tokens,
                                                  int nh, int nkv, int hd, int page_size, int64_t kp, int64_t ks, int64_t kh,
                                                  int64_t vp, int64_t vh, int64_t vd, int max_blocks, int num_splits,
                                                  int chunk, int waves, float scale, int window, int page_run, float softcap,
-                                                 int sink, const float* sinks, const float* slopes, hipStream_t stream) {
+                                                 int sink, const float* sinks, const float* slopes, const float* gate,
+                                                 int64_t gate_stride, hipStream_t stream) {
   if (softcap < 0.f) return TS_BAD_SHAPE;
   return launch_decode(out, part_o, part_ml, q, k_cache, v_cache, block_tables, seq_of_token, positions, num_tokens, nh, nkv, hd,
                        page_size, kp, ks, kh, vp, vh, vd, max_blocks, num_splits, chunk, waves, scale, window, page_run, 1,
-                       true, softcap, sink || sinks, sinks, slopes, stream);
+                       true, softcap, sink || sinks, sinks, slopes, gate, gate_stride, stream);
 }

@@ -267,6 +267,12 @@ static __device__ __forceinline__ void use_tile_auto(const KVTile<HD>& T, int kb
 // [tokens, nh, num_splits, 2] (reference maximum in units of log2, sum), over the chunks that hold
 // keys visible from positions[t] (defined in attention_decode.hip). `sink`: the softmax has one more in its
 // denominator (a key of score 0 without a value, or of score sinks[head] where `sinks` is given), added once, here.
+// `gate` (float [tokens, >= nh hd], rows `gate_stride` apart): the row leaves multiplied by sigmoid(gate).
+static __device__ __forceinline__ float ts_out_gate(const float* __restrict__ gate, int64_t at) {
+  return gate ? 1.0f / (1.0f + expf(-gate[at])) : 1.0f;
+}
+
 int ts_launch_attention_combine(void* out, const float* part_o, const float* part_ml, const int32_t* positions,
                                 int num_tokens, int nh, int hd, int num_splits, int chunk, int window,
-                                hipStream_t stream, int sink = 0, const float* sinks = nullptr);
+                                hipStream_t stream, int sink = 0, const float* sinks = nullptr, const float* gate = nullptr,
+                                int64_t gate_stride = 0);

@@ -51,7 +51,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
              int page_shift, int page_run, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
              float scale2, int window, float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits,
              int chunk, int split, float cap_in, float cap_out, int sink, const float* __restrict__ sinks,
-             const float* __restrict__ slopes) {
+             const float* __restrict__ slopes, const float* __restrict__ gate, int64_t gate_stride) {
   constexpr int NC = HD / 32, NDB = HD / 16;   // operand registers of a 32-key step: 2 NC of K, NDB of V
   auto& stage = lds.stage;
   auto& wg_range = lds.range;
@@ -314,7 +314,11 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
         const float inv = 1.0f / lj;
         bf16_t* orow = out + ((int64_t)(t0 + rtk) * nh + (int64_t)kvh * G + rhh) * HD;
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) orow[16 * db + r] = f2bf(o[j][db][i] * inv);
+        for (int db = 0; db < NDB; ++db) {
+          float y = o[j][db][i] * inv;
+          if (GENERAL) y *= ts_out_gate(gate, (int64_t)(t0 + rtk) * gate_stride + ((int64_t)kvh * G + rhh) * HD + 16 * db + r);
+          orow[16 * db + r] = f2bf(y);
+        }
       }
     }
 }
@@ -329,7 +333,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
                          int64_t vp, int64_t vh, int64_t vd, int max_blocks, float scale2, int window,
                          float* __restrict__ part_o, float* __restrict__ part_ml, int num_splits, int chunk,
                          float cap_in, float cap_out, int sink, const float* __restrict__ sinks,
-                         const float* __restrict__ slopes) {
+                         const float* __restrict__ slopes, const float* __restrict__ gate, int64_t gate_stride) {
   __shared__ PrefillLds<HD> lds;
   // die = workgroup index mod 8. The dies form `groups` groups of `dies_per_group`, the heads as
   // many groups of `heads_per_group`; a group's (tile, head) pairs go round its dies, long tiles first.
@@ -340,7 +344,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q,
   const int kvh = (die / dies_per_group) * heads_per_group + item % heads_per_group;
   prefill_tile<HD, RT, PRE_WAVES, WHOLE, GENERAL>(lds, tile, kvh, out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, nh,
                        G, page_size, page_shift, page_run, kp, ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml,
-                       num_splits, chunk, blockIdx.y, cap_in, cap_out, sink, sinks, slopes);
+                       num_splits, chunk, blockIdx.y, cap_in, cap_out, sink, sinks, slopes, gate, gate_stride);
 }
 
 // Keys: rows dense in head_dim, strides kp/ks/kh (page, slot, head). Values: transposed pages,
@@ -357,8 +361,9 @@ static int launch_prefill(void* out, const void* q, const void* k_cache, const v
                           int64_t ks, int64_t kh, int64_t vp, int64_t vh, int64_t vd, int max_blocks,
                           float scale, int window, int first_token, int num_tokens, int num_splits,
                           int chunk, float* part_o, float* part_ml, int page_run, bool general, float softcap, int sink,
-                          const float* sinks, const float* slopes, hipStream_t stream) {
+                          const float* sinks, const float* slopes, const float* gate, int64_t gate_stride, hipStream_t stream) {
   if (num_tiles <= 0) return TS_OK;
+  if (gate && (!general || gate_stride < (int64_t)nh * hd)) return TS_BAD_SHAPE;
   if (general && (page_size % 32 || softcap < 0.f)) return TS_BAD_SHAPE;     // (the general variant walks whole steps only)
   const float log2e = 1.44269504088896340736f;
   const float cap_in = softcap > 0.f ? scale / softcap : 0.f, cap_out = softcap * log2e;
@@ -393,7 +398,8 @@ static int launch_prefill(void* out, const void* q, const void* k_cache, const v
   attn_prefill_mfma_kernel<HH, RR, WW, PP, GG><<<grid, WW * TS_WAVE, 0, stream>>>(                              \
       (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,             \
       seq_of_token, positions, tiles, num_tiles, nh, G, dies_per_group, heads_per_group, page_size, page_shift, page_run, kp,  \
-      ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml, num_splits, chunk, cap_in, cap_out, sink, sinks, slopes)
+      ks, kh, vp, vh, vd, max_blocks, scale2, window, part_o, part_ml, num_splits, chunk, cap_in, cap_out, sink, sinks, slopes, \
+      gate, gate_stride)
 #define TS_PRE_RT(HH)                                                                                           \
   if (rt == 1) { TS_PRE_W(HH, 1, 4) } else if (rt == 2) { TS_PRE_W(HH, 2, 4) } else { TS_PRE_W(HH, 4, 4) }
 #define TS_PRE_RT8(HH)                                                                                          \
@@ -423,7 +429,8 @@ static int launch_prefill(void* out, const void* q, const void* k_cache, const v
   return ts_launch_attention_combine((bf16_t*)out + skip * hd, part_o + skip * num_splits * hd,
                                      part_ml + skip * num_splits * 2, positions + first_token,
                                      num_tokens - first_token, nh, hd, num_splits, chunk, window, stream, general ? sink : 0,
-                                     general ? sinks : nullptr);
+                                     general ? sinks : nullptr, gate ? gate + (int64_t)first_token * gate_stride : nullptr,
+                                     gate_stride);
 }
 
 extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
@@ -435,13 +442,14 @@ extern "C" int ts_paged_attention_prefill(void* out, const void* q, const void* 
                                           int chunk, float* part_o, float* part_ml, int page_run, hipStream_t stream) {
   return launch_prefill(out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, num_tiles, tile_tokens, waves, nh,
                         nkv, hd, page_size, kp, ks, kh, vp, vh, vd, max_blocks, scale, window, first_token, num_tokens,
-                        num_splits, chunk, part_o, part_ml, page_run, false, 0.f, 0, nullptr, nullptr, stream);
+                        num_splits, chunk, part_o, part_ml, page_run, false, 0.f, 0, nullptr, nullptr, nullptr, 0, stream);
 }
 
 // The same with capped scores (softcap > 0: cap * tanh(score / cap)), a sink (one more in the softmax's
 // denominator; `sinks`, float [nh], if given: exp(sinks[head]) more instead), a penalty of slopes[head] (float [nh],
 // if given) per position of distance taken off every score, and weights carried in two bfloat16 terms; pages of a
-// multiple of 32 keys.
+// multiple of 32 keys. `gate` (float [tokens, >= nh hd], rows gate_stride apart; may be null): the output leaves
+// multiplied by sigmoid(gate).
 extern "C" int ts_paged_attention_prefill_general(void* out, const void* q, const void* k_cache, const void* v_cache,
                                                   const int32_t* block_tables, const int32_t* seq_of_token,
                                                   const int32_t* positions, const int32_t* tiles, int num_tiles,
@@ -450,8 +458,10 @@ extern "C" int ts_paged_attention_prefill_general(void* out, const void* q, cons
                                                   int max_blocks, float scale, int window, int first_token,
                                                   int num_tokens, int num_splits, int chunk, float* part_o,
                                                   float* part_ml, int page_run, float softcap, int sink,
-                                                  const float* sinks, const float* slopes, hipStream_t stream) {
+                                                  const float* sinks, const float* slopes, const float* gate,
+                                                  int64_t gate_stride, hipStream_t stream) {
   return launch_prefill(out, q, k_cache, v_cache, block_tables, seq_of_token, positions, tiles, num_tiles, tile_tokens, waves, nh,
                         nkv, hd, page_size, kp, ks, kh, vp, vh, vd, max_blocks, scale, window, first_token, num_tokens,
-                        num_splits, chunk, part_o, part_ml, page_run, true, softcap, sink || sinks, sinks, slopes, stream);
+                        num_splits, chunk, part_o, part_ml, page_run, true, softcap, sink || sinks, sinks, slopes, gate, gate_stride,
+                        stream);
 }

@@ -164,27 +164,6 @@ extern "C" int ts_embedding_dyt_stream(float* out, const void* table, int dtype,
   return ts_check_launch();
 }
 
-// x *= sigmoid(gate), element by element: x [n, width] as stored, gate 32-bit rows `gate_stride` apart.
-__global__ void __launch_bounds__(DT_THREADS)
-sigmoid_gate_kernel(void* __restrict__ x, int code, const float* __restrict__ gate, int64_t gate_stride, int width, int64_t total) {
-  const int64_t at = (int64_t)blockIdx.x * DT_THREADS + threadIdx.x;
-  if (at >= total) return;
-  const int64_t t = at / width;
-  const float g = gate[t * gate_stride + (at - t * width)];
-  dt_store(x, code, at, dt_load(x, code, at) / (1.0f + expf(-g)));
-}
-
-extern "C" int ts_sigmoid_gate(void* x, int dtype, const float* gate, int64_t gate_stride, int n, int width, hipStream_t stream) {
-  if (n <= 0) return TS_OK;
-  if (width <= 0 || gate_stride < width) return TS_BAD_SHAPE;
-  if (dtype & ~1) return TS_BAD_DTYPE;
-  const int64_t total = (int64_t)n * width;
-  const int64_t blocks = (total + DT_THREADS - 1) / DT_THREADS;
-  if (blocks > 0x7fffffff) return TS_BAD_SHAPE;
-  sigmoid_gate_kernel<<<(unsigned)blocks, DT_THREADS, 0, stream>>>(x, dtype, gate, gate_stride, width, total);
-  return ts_check_launch();
-}
-
 // The capped gated unit between the two projections of a feed-forward: from a row [gate | up] of 32-bit (or
 // stored) sums, g = min(gate, limit), u = clamp(up, -limit, limit), y = g sigmoid(slope g) (u + 1).
 // limit <= 0: no cap. Rows may be picked through `row_stride` (a row of the operand may be wider than 2 ff).

@@ -53,10 +53,9 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_paged_attention_decode": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, i, f,
                                       i, i, i, p],
         "ts_paged_attention_decode_general": [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, i, i, i, f,
-                                              i, i, f, i, p, p, p],
-        "ts_sigmoid_gate": [p, i, p, i64, i, i, p],
+                                              i, i, f, i, p, p, p, i64, p],
         "ts_paged_attention_prefill_general": [p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i, f, i, i, i,
-                                               i, i, p, p, i, f, i, p, p, p],
+                                               i, i, p, p, i, f, i, p, p, p, i64, p],
         "ts_attention_combine": [p, p, p, p, i, i, i, i, i, i, p],
         "ts_gemm_exact": [p, p, p, i, i, i, i64, i64, i64, i, i, p],
         "ts_sample": [p, p, p, p, p, p, u64, i, i, i64, p],
@@ -373,7 +372,8 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
                            chunk: int | None = None, waves: int | None = None,
                            out: torch.Tensor | None = None, pages_per_entry: int = 1,
                            leave_split: bool = False, softcap: float = 0.0, sink: bool = False,
-                           sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None
+                           sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None,
+                           gate: torch.Tensor | None = None
                            ) -> "torch.Tensor | SplitAttention":
     """Split-key attention on the matrix cores for tokens that each bring one query (bfloat16,
     values in transposed pages). Every position in `positions` must lie inside the pages its row
@@ -385,7 +385,7 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     denominator; weights carried in two bfloat16 terms), which always combines; so do `sinks` (float32
     [heads]: exp(sinks[h]) in the denominator instead of 1) and `slopes` (float32 [heads]: slopes[h] times
     the distance between the query's position and the key's is taken off every score)."""
-    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, sinks, slopes)
+    _gpu(q, k_cache, v_cache, block_tables, seq_of_token, positions, sinks, slopes, gate)
     _check_head_vectors(q.shape[1], sinks, slopes)
     _need(q.dim() == 3 and q.is_contiguous(), "q must be contiguous [tokens, heads, head_dim]")
     T, nh, hd = q.shape
@@ -411,7 +411,8 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     if splits > 1:
         part_o = torch.empty((T, nh, splits, hd), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nh, splits, 2), dtype=torch.float32, device=q.device)
-    general = softcap > 0 or sink or sinks is not None or slopes is not None
+    general = softcap > 0 or sink or sinks is not None or slopes is not None or gate is not None
+    gate_stride = _check_gate(gate, q.shape[0], q.shape[1] * q.shape[2])
     leave_split = leave_split and not general and out is None and 1 < splits <= SPLIT_ATTENTION_MAX_CHUNKS
     out = None if leave_split else _out_like(q, out)
     if general:
@@ -419,7 +420,8 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
             _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
             _ptr(seq_of_token), _ptr(positions), T, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3],
             v_cache.stride(0), v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], splits, chunk, waves,
-            float(scale), int(window), _page_run(pages_per_entry), float(softcap), int(sink), _ptr(sinks), _ptr(slopes), _stream()))
+            float(scale), int(window), _page_run(pages_per_entry), float(softcap), int(sink), _ptr(sinks), _ptr(slopes),
+            _ptr(gate), gate_stride, _stream()))
         return out
     _run("paged_attention_decode", library().ts_paged_attention_decode(
         _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
@@ -655,7 +657,8 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             window: int = 0, tile_tokens: int | None = None, out: torch.Tensor | None = None,
                             num_splits: int = 1, chunk: int = 0, first_token: int = 0, waves: int = PREFILL_WAVES,
                             pages_per_entry: int = 1, softcap: float = 0.0, sink: bool = False,
-                            sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None) -> torch.Tensor:
+                            sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None,
+                            gate: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of a packed step on the matrix cores (bfloat16, values in transposed pages).
     `tiles` int32 [num_tiles, 2] lists (first token, token count <= tile_tokens) per workgroup,
     every tile inside one request and inside the step (the caller built the list from the step's
@@ -699,10 +702,12 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
             _ptr(tiles), tiles.shape[0], tile_tokens, waves, nh, nkv, hd, k_cache.shape[1], *k_cache.stride()[:3], v_cache.stride(0),
             v_cache.stride(2), v_cache.stride(3), block_tables.shape[1], float(scale), int(window), first_token, T,
             num_splits, chunk, _ptr(part_o), _ptr(part_ml), _page_run(pages_per_entry))
-    if softcap > 0 or sink or sinks is not None or slopes is not None:
+    if softcap > 0 or sink or sinks is not None or slopes is not None or gate is not None:
         _need(k_cache.shape[1] % 32 == 0, "the general variant takes cache pages of a multiple of 32 keys")
+        _gpu(gate)
         _run("paged_attention_prefill_general", library().ts_paged_attention_prefill_general(
-            *args, float(softcap), int(sink), _ptr(sinks), _ptr(slopes), _stream()))
+            *args, float(softcap), int(sink), _ptr(sinks), _ptr(slopes), _ptr(gate),
+            _check_gate(gate, q.shape[0], q.shape[1] * q.shape[2]), _stream()))
     else:
         _run("paged_attention_prefill", library().ts_paged_attention_prefill(*args, _stream()))
     return out
@@ -721,8 +726,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     back to `paged_attention_general`, which is 32-bit throughout. `sinks` / `slopes` (float32 [heads]): learned
     sinks (exp(sinks[h]) in the denominator) and a penalty of slopes[h] per position of distance on every score,
     by the general variants likewise. `gate` (float32 [tokens, heads * value_dim], rows may lie apart): the
-    output is multiplied element by element by sigmoid(gate), by the 32-bit kernel on its way out or by a
-    kernel of its own behind the matrix-core kernels."""
+    output is multiplied element by element by sigmoid(gate) on its way out of whichever kernel writes it."""
     general = softcap > 0 or sink or sinks is not None or slopes is not None or gate is not None
     extra = dict(softcap=softcap, sink=sink, sinks=sinks, slopes=slopes)
     tables = ctx.block_tables[space]
@@ -735,8 +739,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         capacity = tables.shape[1] * table_page
         decode_ok = -(-capacity // 1024) <= MAX_DECODE_SPLITS and q.shape[0] <= MAX_DECODE_TOKENS
         if ctx.max_query_len == 1 and decode_ok:
-            return _gated(paged_attention_decode(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window,
-                                                 pages_per_entry=per_entry, leave_split=leave_split and gate is None, **extra), gate)
+            return paged_attention_decode(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, window,
+                                          pages_per_entry=per_entry, leave_split=leave_split and gate is None, gate=gate, **extra)
         # the one-token requests that lead the step go to the split-key kernel, the rest to the tiles
         cu = ctx.host_cu_seqlens
         lead = 0
@@ -755,11 +759,12 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         out = torch.empty_like(q)
         if lead:
             paged_attention_decode(q[:lead], k_cache, v_cache, tables, ctx.seq_of_token[:lead], ctx.positions[:lead],
-                                   scale, window, out=out[:lead], pages_per_entry=per_entry, **extra)
+                                   scale, window, out=out[:lead], pages_per_entry=per_entry,
+                                   gate=None if gate is None else gate[:lead], **extra)
         splits, chunk = prefill_splits(tiles.shape[0] * nkv, max(ctx.host_context_lens[lead:], default=0))
-        return _gated(paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale,
-                                              window, tile_tokens=tile_tokens, out=out, num_splits=splits, chunk=chunk,
-                                              first_token=cu[lead], waves=waves, pages_per_entry=per_entry, **extra), gate)
+        return paged_attention_prefill(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, tiles, scale,
+                                       window, tile_tokens=tile_tokens, out=out, num_splits=splits, chunk=chunk,
+                                       first_token=cu[lead], waves=waves, pages_per_entry=per_entry, gate=gate, **extra)
     if general or k_cache.shape[3] != v_cache.shape[3]:
         return paged_attention_general(q, k_cache, v_cache, tables, ctx.seq_of_token, ctx.positions, scale, softcap=softcap,
                                        sink=sink, window=window, pages_per_entry=per_entry, sinks=sinks, slopes=slopes, gate=gate)
@@ -1796,22 +1801,6 @@ def _check_gate(gate: torch.Tensor | None, tokens: int, width: int) -> int:
     _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape == (tokens, width) and gate.stride(1) == 1
           and gate.stride(0) >= width, "the gate must be float32 [tokens, heads * value_dim] with contiguous rows")
     return gate.stride(0)
-
-
-def sigmoid_gate_(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
-    """x *= sigmoid(gate) in place, element by element (x [tokens, ...] contiguous, float32 or bfloat16; gate
-    float32 [tokens, width] with contiguous rows that may lie apart)."""
-    _gpu(x, gate)
-    _need(x.is_contiguous(), "the rows to gate must be contiguous")
-    tokens = x.shape[0]
-    width = x.numel() // max(tokens, 1)
-    stride = _check_gate(gate, tokens, width)
-    _run("sigmoid_gate", library().ts_sigmoid_gate(_ptr(x), _code(x.dtype), _ptr(gate), stride, tokens, width, _stream()))
-    return x
-
-
-def _gated(out, gate: torch.Tensor | None):
-    return out if gate is None else sigmoid_gate_(out, gate)
 
 
 # ---- the dynamic-tanh norm ----
