@@ -281,6 +281,22 @@ static __device__ __forceinline__ moe_f32x4 moe_mfma(moe_u32x4 a, moe_u32x4 b, m
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_bf16x8, a), __builtin_bit_cast(moe_bf16x8, b), acc, 0, 0, 0);
 }
 
+// Four adjacent columns of a row, `left` of which exist: one store where all do and the place is whole pieces.
+static __device__ __forceinline__ void moe_store4(float* p, const float (&y)[4], int left) {
+  if (left >= 4 && ((uintptr_t)p & 15) == 0) { *(float4*)p = make_float4(y[0], y[1], y[2], y[3]); return; }
+  for (int c = 0; c < 4 && c < left; ++c) p[c] = y[c];
+}
+static __device__ __forceinline__ void moe_store4(bf16_t* p, const float (&y)[4], int left) {
+  if (left >= 4 && ((uintptr_t)p & 7) == 0) {
+    uint2 v;
+    v.x = (uint32_t)f2bf(y[0]) | ((uint32_t)f2bf(y[1]) << 16);
+    v.y = (uint32_t)f2bf(y[2]) | ((uint32_t)f2bf(y[3]) << 16);
+    *(uint2*)p = v;
+    return;
+  }
+  for (int c = 0; c < 4 && c < left; ++c) p[c] = f2bf(y[c]);
+}
+
 template <int TM, int TN, bool GLU, typename TO>
 __global__ void __launch_bounds__(MOE_THREADS)
 moe_gemm_mfma_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
@@ -347,9 +363,7 @@ moe_gemm_mfma_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const b
         if constexpr (GLU) y[c] = moe_unit(acc[0][j][i][c], acc[1][j][i][c], limit, slope, shift);
         else y[c] = acc[0][j][i][c];
       }
-#pragma unroll
-      for (int c = 0; c < 4; ++c)
-        if (col + c < N) Num<TO>::st(orow + col + c, y[c]);
+      moe_store4(orow + col, y, N - col);
     }
   }
 }
@@ -419,13 +433,13 @@ moe_gemm_stream_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
   if (r >= rows) return;
   TO* orow = out + (int64_t)pair * N;
   const int c0 = n0 + 4 * g;
+  float y[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
-    float y;
-    if constexpr (GLU) y = moe_unit(acc[0][c], acc[1][c], limit, slope, shift);
-    else y = acc[0][c];
-    if (c0 + c < N) Num<TO>::st(orow + c0 + c, y);
+    if constexpr (GLU) y[c] = moe_unit(acc[0][c], acc[1][c], limit, slope, shift);
+    else y[c] = acc[0][c];
   }
+  moe_store4(orow + c0, y, N - c0);
 }
 
 // Tiles of 128 rows, for steps that give an expert hundreds of rows: both operands go through LDS in the order the
@@ -553,17 +567,17 @@ moe_gemm_lds_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf
 #pragma unroll
       for (int j = 0; j < TN / 2; ++j) {
         const int n = n0 + j * 16 + 4 * g;
+        float y[4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
-          if (n + c < N) Num<TO>::st(orow + n + c, moe_unit(acc[j][i][c], acc[j + TN / 2][i][c], limit, slope, shift));
+        for (int c = 0; c < 4; ++c) y[c] = moe_unit(acc[j][i][c], acc[j + TN / 2][i][c], limit, slope, shift);
+        moe_store4(orow + n, y, N - n);
       }
     } else {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int n = n0 + (wn * TN + j) * 16 + 4 * g;
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-          if (n + c < N) Num<TO>::st(orow + n + c, acc[j][i][c]);
+        const float y[4] = {acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]};
+        moe_store4(orow + n, y, N - n);
       }
     }
   }
