@@ -442,8 +442,9 @@ moe_gemm_stream_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
   moe_store4(orow + c0, y, N - c0);
 }
 
-// Tiles of 128 rows, for steps that give an expert hundreds of rows: both operands go through LDS in the order the
-// matrix instruction wants them (lane (r, g) of fragment f: row 16 (f / 2) + r, elements 32 (f % 2) + 8 g .. + 7),
+// Tiles of 128 rows, for steps that give an expert hundreds of rows: both operands go through LDS, fetched a whole
+// 128-byte line of a row by eight threads side by side and read from LDS as the matrix instruction wants them (lane
+// (r, g) of block b and half h: row 16 b + r, elements 32 h + 8 g .. + 7),
 // 64 of K at a time, two k-steps in flight (one in an LDS buffer being multiplied, the next in registers on its way
 // into the other buffer), as in the engine's tiled product for plain matrices; here the rows of x are gathered by
 // pair, the matrix is the tile's expert's, and the rows of y go to their pairs' places. A workgroup of WM x WN
@@ -478,19 +479,29 @@ moe_gemm_lds_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf
   const bf16_t* we = w + (int64_t)e * (GLU ? 2 : 1) * N * K;
   const bf16_t* xp[LX];
   const bf16_t* wp[LW];
+  // (fetching: eight threads side by side take the eight 16-byte pieces of one row's 64 k, a whole line of memory)
+  int place[LX > LW ? LX : LW];
 #pragma unroll
   for (int i = 0; i < LX; ++i) {
-    const int f = (t + THREADS * i) / 64;
-    const int pair = sorted[first + min((f / 2) * 16 + r, rows - 1)];
-    xp[i] = x + (int64_t)(pair / src_div) * K + (f % 2) * 32 + 8 * g;
+    const int row = (t + THREADS * i) / 8, piece = (t + THREADS * i) % 8;
+    const int pair = sorted[first + min(row, rows - 1)];
+    xp[i] = x + (int64_t)(pair / src_div) * K + 8 * piece;
   }
 #pragma unroll
   for (int i = 0; i < LW; ++i) {
-    const int f = (t + THREADS * i) / 64;
-    int col = (f / 2) * 16 + r;
+    const int row = (t + THREADS * i) / 8, piece = (t + THREADS * i) % 8;
+    int col = row;
     if (GLU) col = min(n0 + col % (BN / 2), N - 1) + (col >= BN / 2 ? N : 0);
     else col = min(n0 + col, N - 1);
-    wp[i] = we + (int64_t)col * K + (f % 2) * 32 + 8 * g;
+    wp[i] = we + (int64_t)col * K + 8 * piece;
+  }
+  // (in LDS row R keeps its piece c at place c ^ (R % 8): the eight threads that store a row fill its 128 bytes, and the
+  // lanes that read one piece of eight rows in a row for the matrix instruction find them in eight different places)
+  static_assert(LX == LW, "as many pieces of x as of the matrix a thread");
+#pragma unroll
+  for (int i = 0; i < LX; ++i) {
+    const int row = (t + THREADS * i) / 8, piece = (t + THREADS * i) % 8;
+    place[i] = row * 8 + (piece ^ (row & 7));
   }
   moe_u32x4 sx0[LX], sw0[LW], sx1[LX], sw1[LW];
   moe_f32x4 acc[TN][TM];
@@ -505,14 +516,16 @@ moe_gemm_lds_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf
   } while (0)
 #define MOE_STASH(S)                                                                                      \
   do {                                                                                                    \
-    _Pragma("unroll") for (int i = 0; i < LX; ++i) lds[S][t + THREADS * i] = sx##S[i];                    \
-    _Pragma("unroll") for (int i = 0; i < LW; ++i) lds[S][FX * 64 + t + THREADS * i] = sw##S[i];          \
+    _Pragma("unroll") for (int i = 0; i < LX; ++i) lds[S][place[i]] = sx##S[i];                           \
+    _Pragma("unroll") for (int i = 0; i < LW; ++i) lds[S][FX * 64 + place[i]] = sw##S[i];                 \
   } while (0)
 #define MOE_MULTIPLY(S)                                                                                   \
   _Pragma("unroll") for (int h = 0; h < 2; ++h) {                                                         \
     moe_u32x4 fx[TM], fw[TN];                                                                             \
-    _Pragma("unroll") for (int i = 0; i < TM; ++i) fx[i] = lds[S][((wm * TM + i) * 2 + h) * 64 + lane];   \
-    _Pragma("unroll") for (int j = 0; j < TN; ++j) fw[j] = lds[S][FX * 64 + ((wn * TN + j) * 2 + h) * 64 + lane]; \
+    _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                        \
+      fx[i] = lds[S][((wm * TM + i) * 16 + r) * 8 + ((4 * h + g) ^ (r & 7))];                             \
+    _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                        \
+      fw[j] = lds[S][FX * 64 + ((wn * TN + j) * 16 + r) * 8 + ((4 * h + g) ^ (r & 7))];                   \
     _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                        \
       _Pragma("unroll") for (int i = 0; i < TM; ++i) acc[j][i] = moe_mfma(fw[j], fx[i], acc[j][i]);       \
   }
