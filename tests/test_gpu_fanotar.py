@@ -512,6 +512,32 @@ def test_mixed_batches_on_pages_and_slots_used_again(case, dtype):
     assert rep.manager.num_available_blocks() == rep.manager.num_blocks
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompts_whole_and_in_long_portions(case, dtype):
+    """Steps of hundreds of tokens take kernels of their own (heads and values behind the convolution in 16-byte
+    pieces and tiles, experts on wide tiles): a prompt of 520 tokens whole, and cut where the second portion
+    starts in the middle of a page, beside a short request."""
+    name, folder, config, _, oracle, _ = case
+    long, short = prompt(321, 520, config.vocab), prompt(322, 40, config.vocab)
+    rows = [oracle.logits(long), oracle.logits(short)]
+    rep = replayer(folder, dtype, 640)
+    marks = [0, 1, 255, 256, 257, 300, 518, 519]
+    got = {}
+    logits = rep.step([{"id": "w", "tokens": long, "want": marks}], ["w"])
+    for j, pos in enumerate(marks):
+        got[(0, pos)] = logits[j]
+    check(got, rows, dtype)
+    got = {}
+    logits = rep.step([{"id": "a", "tokens": long[:263], "want": [0, 262]}, {"id": "b", "tokens": short[:7], "want": [6]}], [])
+    got[(0, 0)], got[(0, 262)], got[(1, 6)] = logits[0], logits[1], logits[2]
+    logits = rep.step([{"id": "b", "tokens": short[7:], "want": [0, 32]}, {"id": "a", "tokens": long[263:], "want": [0, 1, 37, 256]}], ["a", "b"])
+    got[(1, 7)], got[(1, 39)] = logits[0], logits[1]
+    for j, pos in enumerate([263, 264, 300, 519]):
+        got[(0, pos)] = logits[2 + j]
+    check(got, rows, dtype)
+    assert rep.manager.num_available_blocks() == rep.manager.num_blocks
+
+
 def test_a_batch_equals_each_request_alone_in_float32(case):
     """float32: the logits of a request do not depend on what else is in the batch, beyond rounding."""
     name, folder, config, prompts, oracle, rows = case
